@@ -38,6 +38,10 @@ class PositionSpec:
     theta: float = 10000.0
     style: str = "half"
     kind: str = "rope"
+    # (factor, low, high, original) or None: frequencies whose wavelength exceeds original/low
+    # are divided by factor, those below original/high stay, and between the two the share of
+    # the unscaled frequency grows linearly in original/wavelength from 0 to 1
+    scaling: Optional[Tuple[float, float, float, float]] = None
 
 
 @dataclass(frozen=True)
@@ -173,7 +177,9 @@ class NormedAttentionSpec:
     that are rotated, in pairs (i, i + rot_dims/2), by position * rot_base^(-2i/rot_dims); 0 =
     no rotation. value_mix: None; "source" = this mixer's values are kept for the step;
     "mix" = v <- (1 - lambda) v + lambda * (the source's values of the same token), lambda a
-    learned number, and the mixed v is what the cache holds."""
+    learned number, and the mixed v is what the cache holds. qk_norm_per_head: every head of q
+    and of k is normed on its own, with ONE weight of the head's width for all heads of q and one
+    for those of k. rot_scaling: see ``PositionSpec.scaling``."""
     hidden: int
     num_heads: int
     num_kv_heads: int
@@ -187,6 +193,8 @@ class NormedAttentionSpec:
     value_mix: Optional[str] = None
     window: Optional[int] = None
     kind: str = "attention_normed"
+    qk_norm_per_head: bool = False
+    rot_scaling: Optional[Tuple[float, float, float, float]] = None
 
 
 @dataclass(frozen=True)
@@ -304,6 +312,16 @@ class RoutedMLPSpec:
     shared_intermediate: Optional[int] = None
     shared_gate: bool = True
     kind: str = "routed_mlp"
+    # router_bias: a learned number per expert is added to the router's logits.
+    # form "mlp": down(act(up(h))). form "limited_glu": an expert has a gate and an up matrix,
+    # g = min(gate(h), limit), u = clamp(up(h), -limit, limit), down(g * sigmoid(gate_slope * g)
+    # * (u + up_shift)); ``activation`` is not used then. shared_limit: the shared expert's limit.
+    router_bias: bool = False
+    form: str = "mlp"
+    limit: float = 0.0
+    shared_limit: float = 0.0
+    gate_slope: float = 1.702
+    up_shift: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -367,3 +385,57 @@ class SandwichBlockSpec:
     hidden: int = 0
     layer_scale: bool = True
     kind: str = "sandwich"
+
+
+# ---------------------------------------------------------------------------------------------
+# Parts that the Luduvik decoder added; as above, every size and constant is a field.
+
+@dataclass(frozen=True)
+class DecayLinearAttentionSpec:
+    """Linear attention with ONE fixed decay per head and no softmax or denominator: per head a
+    matrix state S [key_dim, value_dim], S_t = decay_h S_{t-1} + k_t v_t^T, o_t = S_t^T q_t.
+
+    input_activation: None, or "silu" applied to the q, k and v projections. rot_dims: the first
+    coordinates of every head of q and k that are rotated in pairs (i, i + rot_dims/2) by position
+    * rot_base^(-2i/rot_dims) (0: none; rot_scaling as ``PositionSpec.scaling``). key_scale: k is
+    multiplied by it after the rotation. head_norm "per_head": every head's readout is divided by
+    its root mean square; "all_heads": the concatenated heads are normed together. norm_weight:
+    the norm has a learned weight per channel. gate_activation: the normed readout is multiplied
+    by silu or sigmoid of a gate projection, then projected."""
+    hidden: int
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    decays: Tuple[float, ...]
+    eps: float
+    input_activation: Optional[str] = None
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: Optional[Tuple[float, float, float, float]] = None
+    key_scale: float = 1.0
+    head_norm: str = "per_head"
+    norm_weight: bool = False
+    gate_activation: str = "silu"
+    kind: str = "decay_linear_attention"
+
+
+@dataclass(frozen=True)
+class BranchMeanSpec:
+    """Several mixers side by side that read the same rows: the result is the mean of their
+    results, each first RMS-normed over the model width with a weight vector of its own.
+    names[i] prefixes the parameters of branches[i]."""
+    hidden: int
+    eps: float
+    branches: Tuple[object, ...]
+    names: Tuple[str, ...]
+    kind: str = "branch_mean"
+
+
+@dataclass(frozen=True)
+class ParallelBlockSpec:
+    """h = norm1(x); x += mixer(h) + ffn(h): one norm, both sublayers read its rows.
+    ffn None: the block has the mixer only."""
+    norm1: object
+    mixer: object
+    ffn: object = None
+    kind: str = "parallel_prenorm"

@@ -17,8 +17,8 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     float eps, int normed, const float* __restrict__ angles, int rot,
     const float* __restrict__ lambda, const T* __restrict__ v_first, T* __restrict__ v_keep,
     const int* __restrict__ dest, T* __restrict__ kcache, T* __restrict__ vcache,
-    int nh, int nkv, int dk, int dv, int dvs) {
-  extern __shared__ float buf[];          // [nh*dk + nkv*dk]
+    int nh, int nkv, int dk, int dv, int dvs, int k_inplace) {
+  extern __shared__ float buf[];          // [nh*dk + nkv*dk], then a factor per head [nh + nkv]
   __shared__ float red[8];
   const int t = blockIdx.x;
   T* row = qkv + (size_t)t * stride;
@@ -48,9 +48,21 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   }
   __syncthreads();
   float fq = 1.f, fk = 1.f;
-  if (normed) {
+  if (normed == 1) {
     fq = rsqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps);
     fk = rsqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps);
+  }
+  // normed == 2: every head of q and of k has a factor of its own; the weights wq, wk are then
+  // [dk], shared by the heads. A wave takes heads in turn.
+  float* hf = buf + nq + nk;
+  if (normed == 2) {
+    for (int hd = threadIdx.x / TA_WAVE; hd < nh + nkv; hd += 4) {
+      float ss = 0.f;
+      for (int c = threadIdx.x % TA_WAVE; c < dk; c += TA_WAVE) ss += buf[hd * dk + c] * buf[hd * dk + c];
+      ss = wave_sum(ss);
+      if (threadIdx.x % TA_WAVE == 0) hf[hd] = rsqrtf(ss / (float)dk + eps);
+    }
+    __syncthreads();
   }
   const int half = rot / 2;
   const float* ang = angles ? angles + (size_t)t * half * 2 : nullptr;
@@ -62,7 +74,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     const bool is_q = i < nq;
     const int j = is_q ? i : i - nq;
     const int head = j / dk, c = j - head * dk;
-    const float f = is_q ? fq : fk;
+    const float f = normed == 2 ? hf[i / dk] : is_q ? fq : fk;
     const float* w = is_q ? wq : wk;
     const bool turns = ang != nullptr && c < rot;
     const int pi = turns ? (c < half ? c : c - half) : 0;
@@ -70,13 +82,14 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     const float cs = ang ? ang[2 * pi] : 1.f, sn = ang ? ang[2 * pi + 1] : 0.f;
     float wv = 1.f, wo = 1.f;
     if (normed) {                     // the same for every thread
-      wv = w[j];
-      wo = w[j + shift];
+      const int jw = normed == 2 ? c : j;
+      wv = w[jw];
+      wo = w[jw + shift];
     }
     float v = buf[i] * f * wv;
     const float o = buf[i + shift] * f * wo;
     if (turns) v = c < half ? v * cs - o * sn : v * cs + o * sn;
-    if (is_q) {
+    if (is_q || k_inplace) {
       row[i] = from_f32<T>(v);
     } else if (dest) {
       kcache[(((size_t)page * nkv + head) * TA_PAGE + off) * dk + c] = from_f32<T>(v);
@@ -150,8 +163,8 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(
     float eps, int normed, const float* __restrict__ angles, int rot,
     const float* __restrict__ lambda, const T* __restrict__ v_first, T* __restrict__ v_keep,
     const int* __restrict__ dest, T* __restrict__ kcache, T* __restrict__ vcache,
-    int nh, int nkv, int dk, int dv, int dvs) {
-  extern __shared__ float buf[];          // [nh*dk + nkv*dk]
+    int nh, int nkv, int dk, int dv, int dvs, int k_inplace) {
+  extern __shared__ float buf[];          // [nh*dk + nkv*dk], then a factor per head [nh + nkv]
   __shared__ float red[8];
   const int t = blockIdx.x;
   T* row = qkv + (size_t)t * stride;
@@ -177,9 +190,21 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(
   }
   __syncthreads();
   float fq = 1.f, fk = 1.f;
-  if (normed) {
+  if (normed == 1) {
     fq = rsqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps);
     fk = rsqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps);
+  }
+  // normed == 2: every head of q and of k has a factor of its own; the weights wq, wk are then
+  // [dk], shared by the heads. A wave takes heads in turn.
+  float* hf = buf + nq + nk;
+  if (normed == 2) {
+    for (int hd = threadIdx.x / TA_WAVE; hd < nh + nkv; hd += 4) {
+      float ss = 0.f;
+      for (int c = threadIdx.x % TA_WAVE; c < dk; c += TA_WAVE) ss += buf[hd * dk + c] * buf[hd * dk + c];
+      ss = wave_sum(ss);
+      if (threadIdx.x % TA_WAVE == 0) hf[hd] = rsqrtf(ss / (float)dk + eps);
+    }
+    __syncthreads();
   }
   const int half = rot / 2;
   const float* ang = angles ? angles + (size_t)t * half * 2 : nullptr;
@@ -189,7 +214,7 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(
     const bool is_q = i < nq;
     const int j = is_q ? i : i - nq;
     const int head = j / dk, c = j - head * dk;            // the piece lies inside one head
-    const float f = is_q ? fq : fk;
+    const float f = normed == 2 ? hf[i / dk] : is_q ? fq : fk;
     const float* w = is_q ? wq : wk;
     const bool turns = ang != nullptr && c < rot;          // and wholly inside or outside the rotation
     const int shift = turns ? (c < half ? half : -half) : 0;
@@ -197,8 +222,9 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) wv[e] = wo[e] = cs[e] = 1.f, sn[e] = 0.f;
     if (normed) {
-      Eight<float>::load(w + j, wv);
-      Eight<float>::load(w + j + shift, wo);
+      const int jw = normed == 2 ? c : j;
+      Eight<float>::load(w + jw, wv);
+      Eight<float>::load(w + jw + shift, wo);
     }
     if (turns) {
       float a[8], b[8];
@@ -217,7 +243,7 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(
       const float v = buf[i + e] * f * wv[e], o = buf[i + shift + e] * f * wo[e];
       out[e] = turns ? (c < half ? v * cs[e] - o * sn[e] : v * cs[e] + o * sn[e]) : v;
     }
-    if (is_q) Eight<T>::store(row + i, out);
+    if (is_q || k_inplace) Eight<T>::store(row + i, out);
     else if (dest) Eight<T>::store(kcache + (((size_t)page * nkv + head) * TA_PAGE + off) * dk + c, out);
   }
   const float lam = lambda ? lambda[0] : 0.f;
@@ -239,7 +265,9 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(
   }
 }
 
-// qkv: [nt, stride] rows of [nh*dk | nkv*dk | nkv*dv]. wq [nh*dk], wk [nkv*dk] (used when normed).
+// qkv: [nt, stride] rows of [nh*dk | nkv*dk | nkv*dv]. normed 1: wq [nh*dk], wk [nkv*dk], one norm over
+// all heads of q and one over all of k; normed 2: wq, wk [dk], every head normed on its own; 0: no norm.
+// k_inplace (no dest): the keys are written back into their rows as the queries are.
 // angles: [nt, rot/2, 2] (cos, sin) or null. lambda: one float on the device, v_first [nt, nkv*dv]
 // (both or neither). v_keep [nt, nkv*dv] or null: receives the unmixed values. dest [nt] or null:
 // page * PAGE + offset of each token in the cache layer.
@@ -247,15 +275,17 @@ extern "C" int ta_qk_prepare(hipStream_t stream, int dtype, void* qkv, int strid
                              const float* wk, float eps, int normed, const float* angles, int rot,
                              const float* lambda, const void* v_first, void* v_keep, const int* dest,
                              void* kcache, void* vcache, int nt, int nh, int nkv, int dk, int dv,
-                             int dvs) {
+                             int dvs, int k_inplace) {
   TA_REQUIRE(nt >= 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "ta_qk_prepare: bad sizes");
+  TA_REQUIRE(normed >= 0 && normed <= 2, "ta_qk_prepare: unknown norm mode %d", normed);
+  TA_REQUIRE(!(k_inplace && dest), "ta_qk_prepare: keys go back in place or to the cache, not both");
   TA_REQUIRE(stride >= (nh + nkv) * dk + nkv * dv, "ta_qk_prepare: row stride %d too small", stride);
   TA_REQUIRE(rot >= 0 && rot <= dk && rot % 2 == 0, "ta_qk_prepare: %d rotated coordinates of %d", rot, dk);
   TA_REQUIRE((lambda == nullptr) == (v_first == nullptr), "ta_qk_prepare: lambda and v_first go together");
   TA_REQUIRE(!normed || (wq && wk), "ta_qk_prepare: norm weights missing");
   TA_REQUIRE(!dest || (kcache && vcache), "ta_qk_prepare: cache layer missing");
   TA_REQUIRE(dvs >= dv, "ta_qk_prepare: cache rows of %d cannot hold values of %d", dvs, dv);
-  const size_t lds = (size_t)(nh + nkv) * dk * sizeof(float);
+  const size_t lds = ((size_t)(nh + nkv) * dk + nh + nkv) * sizeof(float);
   TA_REQUIRE(lds <= 60000, "ta_qk_prepare: %d + %d heads of %d do not fit", nh, nkv, dk);
   if (nt == 0) return 0;
   if (rot == 0) angles = nullptr;
@@ -267,21 +297,21 @@ extern "C" int ta_qk_prepare(hipStream_t stream, int dtype, void* qkv, int strid
     if (dtype == TA_F32)
       qk_prepare_vec_kernel<float><<<nt, 256, lds, stream>>>(
           (float*)qkv, stride, wq, wk, eps, normed, angles, rot, lambda, (const float*)v_first, (float*)v_keep,
-          dest, (float*)kcache, (float*)vcache, nh, nkv, dk, dv, dvs);
+          dest, (float*)kcache, (float*)vcache, nh, nkv, dk, dv, dvs, k_inplace);
     else
       qk_prepare_vec_kernel<bf16_t><<<nt, 256, lds, stream>>>(
           (bf16_t*)qkv, stride, wq, wk, eps, normed, angles, rot, lambda, (const bf16_t*)v_first, (bf16_t*)v_keep,
-          dest, (bf16_t*)kcache, (bf16_t*)vcache, nh, nkv, dk, dv, dvs);
+          dest, (bf16_t*)kcache, (bf16_t*)vcache, nh, nkv, dk, dv, dvs, k_inplace);
     return ta_check_launch("ta_qk_prepare");
   }
   if (dtype == TA_F32)
     qk_prepare_kernel<float><<<nt, 256, lds, stream>>>(
         (float*)qkv, stride, wq, wk, eps, normed, angles, rot, lambda, (const float*)v_first, (float*)v_keep,
-        dest, (float*)kcache, (float*)vcache, nh, nkv, dk, dv, dvs);
+        dest, (float*)kcache, (float*)vcache, nh, nkv, dk, dv, dvs, k_inplace);
   else if (dtype == TA_BF16)
     qk_prepare_kernel<bf16_t><<<nt, 256, lds, stream>>>(
         (bf16_t*)qkv, stride, wq, wk, eps, normed, angles, rot, lambda, (const bf16_t*)v_first, (bf16_t*)v_keep,
-        dest, (bf16_t*)kcache, (bf16_t*)vcache, nh, nkv, dk, dv, dvs);
+        dest, (bf16_t*)kcache, (bf16_t*)vcache, nh, nkv, dk, dv, dvs, k_inplace);
   else
     return ta_fail("ta_qk_prepare: unknown dtype %d", dtype);
   return ta_check_launch("ta_qk_prepare");

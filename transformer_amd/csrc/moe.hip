@@ -22,19 +22,22 @@
 
 // ------------------------------------------------------------------ routing
 // logits: [nt, ld] float32, the first E columns of a row are the router's. mode 0: sigmoid
-// scores; 1: softmax over the experts. renorm: the chosen weights are divided by their sum.
+// scores; 1: softmax over the experts. renorm: the chosen weights are divided by their sum
+// (with mode 1 that is the softmax over the chosen logits alone). bias [E] or null: added to
+// the logits first.
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int ld, int E, int top,
                                                        int mode, int renorm, int* __restrict__ chosen,
-                                                       float* __restrict__ weight) {
+                                                       float* __restrict__ weight,
+                                                       const float* __restrict__ bias) {
   extern __shared__ float sc[];           // [E]
   const size_t t = blockIdx.x;
   const int lane = threadIdx.x;
   float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, logits[t * ld + e]);
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, logits[t * ld + e] + (bias ? bias[e] : 0.f));
   mx = wave_max(mx);
   float sum = 0.f;
   for (int e = lane; e < E; e += 64) {
-    const float z = logits[t * ld + e];
+    const float z = logits[t * ld + e] + (bias ? bias[e] : 0.f);
     const float s = mode == 0 ? 1.0f / (1.0f + expf(-z)) : expf(z - mx);
     sc[e] = s;
     sum += s;
@@ -71,13 +74,18 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
   }
 }
 
-extern "C" int ta_moe_route(hipStream_t stream, const float* logits, int ld, int nt, int E, int top, int mode,
-                            int renorm, int* chosen, float* weight) {
+extern "C" int ta_moe_route_bias(hipStream_t stream, const float* logits, const float* bias, int ld, int nt, int E,
+                                 int top, int mode, int renorm, int* chosen, float* weight) {
   TA_REQUIRE(nt >= 0 && E >= 1 && E <= 8192 && top >= 1 && top <= E && ld >= E && (mode == 0 || mode == 1),
              "ta_moe_route: bad sizes nt=%d experts=%d top=%d ld=%d", nt, E, top, ld);
   if (nt == 0) return 0;
-  moe_route_kernel<<<nt, 64, (size_t)E * sizeof(float), stream>>>(logits, ld, E, top, mode, renorm, chosen, weight);
+  moe_route_kernel<<<nt, 64, (size_t)E * sizeof(float), stream>>>(logits, ld, E, top, mode, renorm, chosen, weight, bias);
   return ta_check_launch("ta_moe_route");
+}
+
+extern "C" int ta_moe_route(hipStream_t stream, const float* logits, int ld, int nt, int E, int top, int mode,
+                            int renorm, int* chosen, float* weight) {
+  return ta_moe_route_bias(stream, logits, nullptr, ld, nt, E, top, mode, renorm, chosen, weight);
 }
 
 // ------------------------------------------------------------------ ordering the pairs by expert
@@ -635,7 +643,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
                                                           const float* __restrict__ weight,
                                                           const float* __restrict__ shared, int planes, size_t plane,
                                                           const float* __restrict__ shared_gate, int gate_ld,
-                                                          float* __restrict__ delta) {
+                                                          float* __restrict__ delta,
+                                                          const float* __restrict__ extra, int xplanes, size_t xplane) {
   extern __shared__ float cmb[];          // [top] rows of the token's pairs, [top] their weights
   int* prow = reinterpret_cast<int*>(cmb);
   float* pw = cmb + top;
@@ -655,6 +664,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
       for (int p = 1; p < planes; ++p) v += shared[t * d + c + p * plane];
       s += sg * v;
     }
+    if (extra)      // what another sublayer adds to the stream beside this one, planes in order
+      for (int p = 0; p < xplanes; ++p) s += extra[t * d + c + p * xplane];
     delta[t * d + c] = s;
   }
 }
@@ -663,12 +674,58 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 // has acted on the inputs. shared (or null): [planes, nt, d] float32 planes that add up to the
 // shared expert's result; shared_gate (or null): its gate's pre-activation, one number per
 // token, element 0 of a row of gate_ld float32. delta: [nt, d] float32.
+// extra (or null): [xplanes, nt, d] float32 planes, ``xplane`` elements apart, added as they are.
+extern "C" int ta_moe_combine_extra(hipStream_t stream, const float* rows, int d, int top, const int* pair_row,
+                                    const float* weight, const float* shared, int planes, long long plane,
+                                    const float* shared_gate, int gate_ld, const float* extra, int xplanes,
+                                    long long xplane, float* delta, int nt) {
+  TA_REQUIRE(nt >= 0 && d > 0 && top >= 1 && planes >= 1 && planes <= TA_MAX_PLANES, "ta_moe_combine: bad sizes");
+  TA_REQUIRE(!extra || (xplanes >= 1 && xplanes <= TA_MAX_PLANES && (xplanes == 1 || xplane > 0)),
+             "ta_moe_combine: %d planes of the further addend", xplanes);
+  if (nt == 0) return 0;
+  moe_combine_kernel<<<nt, 256, (size_t)2 * top * sizeof(float), stream>>>(rows, d, top, pair_row, weight, shared, planes, (size_t)plane,
+                                             shared_gate, gate_ld, delta, extra, xplanes, (size_t)xplane);
+  return ta_check_launch("ta_moe_combine");
+}
+
 extern "C" int ta_moe_combine(hipStream_t stream, const float* rows, int d, int top, const int* pair_row,
                               const float* weight, const float* shared, int planes, long long plane,
                               const float* shared_gate, int gate_ld, float* delta, int nt) {
-  TA_REQUIRE(nt >= 0 && d > 0 && top >= 1 && planes >= 1 && planes <= TA_MAX_PLANES, "ta_moe_combine: bad sizes");
-  if (nt == 0) return 0;
-  moe_combine_kernel<<<nt, 256, (size_t)2 * top * sizeof(float), stream>>>(rows, d, top, pair_row, weight, shared, planes, (size_t)plane,
-                                             shared_gate, gate_ld, delta);
-  return ta_check_launch("ta_moe_combine");
+  return ta_moe_combine_extra(stream, rows, d, top, pair_row, weight, shared, planes, plane, shared_gate, gate_ld,
+                              nullptr, 0, 0, delta, nt);
+}
+
+// ------------------------------------------------------------------ the limited gated activation
+// Rows of [gate | up] (``di`` columns each, ``ld`` elements between rows): g = min(gate, limit),
+// u = clamp(up, -limit, limit), out = g * sigmoid(slope * g) * (u + shift). float32 inside.
+template <typename T>
+__global__ __launch_bounds__(256) void glu_limit_kernel(const T* __restrict__ gu, int ld, T* __restrict__ out, int di,
+                                                        float limit, float slope, float shift) {
+  const size_t t = blockIdx.y;
+  const T* g = gu + t * (size_t)ld;
+  T* o = out + t * (size_t)di;
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < di; i += gridDim.x * 256) {
+    const float a = fminf(to_f32(g[i]), limit);
+    const float u = fminf(fmaxf(to_f32(g[di + i]), -limit), limit);
+    o[i] = from_f32<T>(a / (1.0f + expf(-slope * a)) * (u + shift));
+  }
+}
+
+extern "C" int ta_glu_limit(hipStream_t stream, int dtype, const void* gate_up, int ld, void* out, int nt, int di,
+                            float limit, float slope, float shift) {
+  TA_REQUIRE(nt >= 0 && di > 0 && ld >= 2 * di, "ta_glu_limit: bad sizes nt=%d di=%d ld=%d", nt, di, ld);
+  TA_REQUIRE(limit > 0.f, "ta_glu_limit: the limit must be positive, got %g", (double)limit);
+  for (int t0 = 0; t0 < nt; t0 += 65535) {
+    const int rows = nt - t0 < 65535 ? nt - t0 : 65535;
+    dim3 g((di + 1023) / 1024 < 64 ? (di + 1023) / 1024 : 64, rows);
+    if (dtype == TA_F32)
+      glu_limit_kernel<float><<<g, 256, 0, stream>>>((const float*)gate_up + (size_t)t0 * ld, ld,
+                                                    (float*)out + (size_t)t0 * di, di, limit, slope, shift);
+    else if (dtype == TA_BF16)
+      glu_limit_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)gate_up + (size_t)t0 * ld, ld,
+                                                     (bf16_t*)out + (size_t)t0 * di, di, limit, slope, shift);
+    else
+      return ta_fail("ta_glu_limit: unknown dtype %d", dtype);
+  }
+  return ta_check_launch("ta_glu_limit");
 }

@@ -569,7 +569,7 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
     const T* __restrict__ proj, int stride, int qoff, int koff, int voff, const float* __restrict__ alpha,
     float qscale, float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots,
     int H, int dk, int dv, int col_tiles, size_t plane, float* __restrict__ o_out,
-    const float* __restrict__ bonus) {
+    const float* __restrict__ bonus, const float* __restrict__ head_decay) {
   __shared__ float sq[GLA_TC][GLA_RT], sk[GLA_TC][GLA_RT], sa[GLA_TC][GLA_RT];
   __shared__ float sv[GLA_TC][GLA_CT];
   __shared__ float part[GLA_TC][4][GLA_CT];
@@ -598,6 +598,8 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
       bu[r] = i < dk ? bonus[h * dk + i] : 0.f;
     }
   }
+  // one fixed decay for all key channels of the head (``alpha`` is then not read)
+  const float fixed = head_decay ? head_decay[h] : 0.f;
   // Loads are asked for two chunks ahead (a trip to memory takes longer than a chunk's
   // arithmetic); a position that is not there reads a harmless address and is replaced.
   auto fetch = [&](GlaOperands<GLA_TC>& o, int t0) {
@@ -609,7 +611,7 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
       const int ii = ok ? i : 0;
       const float qv = to_f32(proj[row * stride + qoff + h * dk + ii]);
       const float kv = to_f32(proj[row * stride + koff + h * dk + ii]);
-      const float av = alpha[row * ((size_t)H * dk) + h * dk + ii];
+      const float av = head_decay ? fixed : alpha[row * ((size_t)H * dk) + h * dk + ii];
       o.q[e] = ok ? qv * qscale : 0.f;
       o.k[e] = ok ? kv : 0.f;
       o.a[e] = ok ? av : 1.f;           // a token that is not there leaves S as it is
@@ -718,10 +720,12 @@ static int gla_recurrent_launch(hipStream_t stream, int dtype, int wdtype, const
                                 int qoff, int koff, int voff, const void* low, int low_stride, int aoff, int rank,
                                 const void* a2, const float* a2b, float inv_tau, float qscale, float* alpha,
                                 float* state, const int* cu_q, const int* slots, int batch, int nt, int H, int dk,
-                                int dv, float* o_out, int mode, const float* bonus) {
+                                int dv, float* o_out, int mode, const float* bonus,
+                                const float* head_decay = nullptr) {
   TA_REQUIRE(batch > 0 && batch <= 65535 && H > 0 && H <= 65535 && nt >= batch,
              "ta_gla_recurrent: bad batch %d / heads %d / tokens %d", batch, H, nt);
-  TA_REQUIRE(dk >= 1 && dv >= 1 && rank >= 1 && rank <= 8192, "ta_gla_recurrent: bad widths %d / %d / %d", dk, dv, rank);
+  TA_REQUIRE(dk >= 1 && dv >= 1 && (head_decay || (rank >= 1 && rank <= 8192)),
+             "ta_gla_recurrent: bad widths %d / %d / %d", dk, dv, rank);
   const int parts = (dk + GLA_RT - 1) / GLA_RT, tiles = (dv + GLA_CT - 1) / GLA_CT;
   TA_REQUIRE(parts * tiles <= 65535, "ta_gla_recurrent: heads of %d x %d are too large", dk, dv);
   const int n = H * dk;
@@ -729,7 +733,9 @@ static int gla_recurrent_launch(hipStream_t stream, int dtype, int wdtype, const
   const size_t lds = (size_t)rank * sizeof(float);
 #define GLA_DECAY(T, TW) \
   gla_decay_kernel<T, TW><<<gd, 256, lds, stream>>>((const T*)low, low_stride, aoff, rank, (const TW*)a2, a2b, inv_tau, n, alpha, mode)
-  if (dtype == TA_F32 && wdtype == TA_F32) GLA_DECAY(float, float);
+  if (head_decay) {
+    TA_REQUIRE(dtype == TA_F32 || dtype == TA_BF16, "ta_gla_recurrent: unknown dtype %d", dtype);
+  } else if (dtype == TA_F32 && wdtype == TA_F32) GLA_DECAY(float, float);
   else if (dtype == TA_BF16 && wdtype == TA_BF16) GLA_DECAY(bf16_t, bf16_t);
   else if (dtype == TA_BF16 && wdtype == TA_F32) GLA_DECAY(bf16_t, float);
   else return ta_fail("ta_gla_recurrent: unsupported dtypes %d / %d", dtype, wdtype);
@@ -739,7 +745,8 @@ static int gla_recurrent_launch(hipStream_t stream, int dtype, int wdtype, const
   const bool few = nt <= 8 * batch;         // at most 8 tokens a sequence on average: short chunks
 #define GLA_RUN(T, TC, B)                                                                                   \
   gla_recurrent_kernel<T, TC, B><<<g, 256, 0, stream>>>((const T*)proj, stride, qoff, koff, voff, alpha, qscale, \
-                                                        state, cu_q, slots, H, dk, dv, tiles, plane, o_out, bonus)
+                                                        state, cu_q, slots, H, dk, dv, tiles, plane, o_out, bonus, \
+                                                        head_decay)
   if (bonus) {
     if (dtype == TA_F32) {
       if (few) GLA_RUN(float, 8, true); else GLA_RUN(float, 32, true);
@@ -779,12 +786,25 @@ extern "C" int ta_wkv_recurrent(hipStream_t stream, int dtype, int wdtype, const
                               a2b, 1.0f, 1.0f, alpha, state, cu_q, slots, batch, nt, H, dk, dv, o_out, 1, bonus);
 }
 
+// The recurrence with ONE fixed decay per head, S_t = decay_h S_{t-1} + k_t v_t^T, o_t = S_t^T
+// (qscale q_t): head_decay [H] float32 on the device; q, k, v at element offsets of the rows of
+// ``proj`` as above. No decay input, no scratch for decays.
+extern "C" int ta_decay_recurrent(hipStream_t stream, int dtype, const void* proj, int stride, int qoff, int koff,
+                                  int voff, const float* head_decay, float qscale, float* state, const int* cu_q,
+                                  const int* slots, int batch, int nt, int H, int dk, int dv, float* o_out) {
+  TA_REQUIRE(head_decay != nullptr, "ta_decay_recurrent: the heads' decays are required");
+  return gla_recurrent_launch(stream, dtype, dtype, proj, stride, qoff, koff, voff, nullptr, 0, 0, 0, nullptr,
+                              nullptr, 1.0f, qscale, nullptr, state, cu_q, slots, batch, nt, H, dk, dv, o_out, 0,
+                              nullptr, head_decay);
+}
+
 // ------------------------------------------------------------------ gla: head norm and output gate
 template <typename T>
 __global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o, int parts, size_t plane,
                                                      const T* __restrict__ proj,
                                                      int stride, int goff, const float* __restrict__ w,
-                                                     int wstride, float eps, int H, int dv, T* __restrict__ out) {
+                                                     int wstride, float eps, int H, int dv, T* __restrict__ out,
+                                                     int gate_act) {
   extern __shared__ float row[];          // [dv]
   const size_t t = blockIdx.x;
   const int h = blockIdx.y;
@@ -799,28 +819,39 @@ __global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o
   const float f = rsqrtf(wave_sum(ss) / (float)dv + eps);
   for (int c = threadIdx.x; c < dv; c += 64) {
     const float g = to_f32(proj[t * stride + goff + h * dv + c]);
-    out[t * (size_t)(H * dv) + h * dv + c] = from_f32<T>(row[c] * f * w[h * wstride + c] * (g / (1.0f + expf(-g))));
+    const float sg = 1.0f / (1.0f + expf(-g));
+    const float wc = w ? w[h * wstride + c] : 1.0f;                        // no weight: the plain unit norm
+    out[t * (size_t)(H * dv) + h * dv + c] = from_f32<T>(row[c] * f * wc * (gate_act == 1 ? sg : g * sg));
   }
 }
 
 // o: [parts, nt, H, dv] float32 planes that add up to the readout; the gate's pre-activation sits
 // at element goff of proj, ``stride`` elements between tokens; w [dv] shared by the heads
 // (wstride 0) or [H, dv] (wstride dv); out [nt, H*dv] = rms_norm(o per head) * w * silu(gate).
-extern "C" int ta_gla_out_w(hipStream_t stream, int dtype, const float* o, int parts, const void* proj, int stride,
-                            long long goff, const float* w, int wstride, float eps, int nt, int H, int dv,
-                            void* out) {
+// gate_act 0: silu(gate); 1: sigmoid(gate). w may be null (no weight).
+extern "C" int ta_gla_out_act(hipStream_t stream, int dtype, const float* o, int parts, const void* proj, int stride,
+                              long long goff, const float* w, int wstride, float eps, int nt, int H, int dv,
+                              int gate_act, void* out) {
   TA_REQUIRE(nt >= 0 && H > 0 && H <= 65535 && dv > 0 && dv <= 15000 && parts >= 1, "ta_gla_out: bad sizes");
+  TA_REQUIRE(gate_act == 0 || gate_act == 1, "ta_gla_out: unknown gate activation %d", gate_act);
   TA_REQUIRE(wstride == 0 || wstride == dv, "ta_gla_out: weight rows of %d for heads of %d", wstride, dv);
   if (nt == 0) return 0;
   dim3 g(nt, H);
   const size_t plane = (size_t)nt * H * dv, lds = (size_t)dv * sizeof(float);
   if (dtype == TA_F32)
-    gla_out_kernel<float><<<g, 64, lds, stream>>>(o, parts, plane, (const float*)proj + goff, stride, 0, w, wstride, eps, H, dv, (float*)out);
+    gla_out_kernel<float><<<g, 64, lds, stream>>>(o, parts, plane, (const float*)proj + goff, stride, 0, w, wstride, eps, H, dv, (float*)out, gate_act);
   else if (dtype == TA_BF16)
-    gla_out_kernel<bf16_t><<<g, 64, lds, stream>>>(o, parts, plane, (const bf16_t*)proj + goff, stride, 0, w, wstride, eps, H, dv, (bf16_t*)out);
+    gla_out_kernel<bf16_t><<<g, 64, lds, stream>>>(o, parts, plane, (const bf16_t*)proj + goff, stride, 0, w, wstride, eps, H, dv, (bf16_t*)out, gate_act);
   else
     return ta_fail("ta_gla_out: unknown dtype %d", dtype);
   return ta_check_launch("ta_gla_out");
+}
+
+extern "C" int ta_gla_out_w(hipStream_t stream, int dtype, const float* o, int parts, const void* proj, int stride,
+                            long long goff, const float* w, int wstride, float eps, int nt, int H, int dv,
+                            void* out) {
+  TA_REQUIRE(w != nullptr, "ta_gla_out: the weight is required");
+  return ta_gla_out_act(stream, dtype, o, parts, proj, stride, goff, w, wstride, eps, nt, H, dv, 0, out);
 }
 
 extern "C" int ta_gla_out(hipStream_t stream, int dtype, const float* o, int parts, const void* proj, int stride,

@@ -188,3 +188,57 @@ extern "C" int ta_activation(hipStream_t stream, int dtype, int act, const void*
   }
   return ta_check_launch("ta_activation");
 }
+
+// ------------------------------------------------------------------ the mean of normed branches
+// out[t] = (1/n) * sum over branches b of rms_norm(sum of the planes of delta_b[t], eps) * w_b.
+// A thread owns the same columns in every pass, so the sum over branches needs no exchange; the
+// planes are read a second time (from the caches) once a branch's factor is known.
+struct MeanBranch {
+  const float* delta;     // [planes, nt, d]
+  const float* w;         // [d]
+  long long plane;        // elements between planes
+  int planes;
+};
+struct MeanBranches {
+  MeanBranch b[4];
+};
+
+__global__ __launch_bounds__(256) void normed_mean_kernel(MeanBranches br, int n, float eps, float* __restrict__ out,
+                                                          int d) {
+  __shared__ float red[4];
+  const size_t base = (size_t)blockIdx.x * d;
+  const float inv = 1.0f / (float)n;
+  for (int k = 0; k < n; ++k) {
+    const MeanBranch b = br.b[k];
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < d; c += 256) {
+      float s = b.delta[base + c];
+      for (int p = 1; p < b.planes; ++p) s += b.delta[base + c + p * b.plane];
+      ss += s * s;
+    }
+    const float f = rsqrtf(block_sum4(ss, red) / (float)d + eps);
+    for (int c = threadIdx.x; c < d; c += 256) {
+      float s = b.delta[base + c];
+      for (int p = 1; p < b.planes; ++p) s += b.delta[base + c + p * b.plane];
+      const float v = s * f * b.w[c] * inv;
+      out[base + c] = k == 0 ? v : out[base + c] + v;
+    }
+  }
+}
+
+// deltas[i]: [planes[i], nt, d] float32, ``plane[i]`` elements apart; ws[i]: [d]; out [nt, d].
+extern "C" int ta_normed_mean(hipStream_t stream, int n, const float* const* deltas, const int* planes,
+                              const long long* plane, const float* const* ws, float eps, float* out, int nt, int d) {
+  TA_REQUIRE(n >= 1 && n <= 4, "ta_normed_mean: %d branches (1 to 4 are taken)", n);
+  TA_REQUIRE(nt >= 0 && d > 0, "ta_normed_mean: bad sizes nt=%d d=%d", nt, d);
+  MeanBranches br;
+  for (int i = 0; i < 4; ++i) br.b[i] = MeanBranch{nullptr, nullptr, 0, 1};
+  for (int i = 0; i < n; ++i) {
+    TA_REQUIRE(deltas[i] && ws[i] && planes[i] >= 1 && planes[i] <= TA_MAX_PLANES,
+               "ta_normed_mean: branch %d: %d planes", i, planes[i]);
+    br.b[i] = MeanBranch{deltas[i], ws[i], plane[i], planes[i]};
+  }
+  if (nt == 0) return 0;
+  normed_mean_kernel<<<nt, 256, 0, stream>>>(br, n, eps, out, d);
+  return ta_check_launch("ta_normed_mean");
+}

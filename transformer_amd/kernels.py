@@ -977,13 +977,16 @@ def qk_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_dim: in
                angles: Optional[torch.Tensor], rot: int, mix: Optional[torch.Tensor] = None,
                v_first: Optional[torch.Tensor] = None, v_keep: Optional[torch.Tensor] = None,
                dest: Optional[torch.Tensor] = None, kcache: Optional[torch.Tensor] = None,
-               vcache: Optional[torch.Tensor] = None) -> torch.Tensor:
+               vcache: Optional[torch.Tensor] = None, per_head: bool = False,
+               k_inplace: bool = False) -> torch.Tensor:
     """On rows [q | k | v] of ``qkv`` (nh*dk, nkv*dk, nkv*dv columns): RMS norm of q and of k
-    over all their heads at once (weights given: else none), rotation of the first ``rot``
+    over all their heads at once (weights given: else none; ``per_head``: every head on its own,
+    the weights then have the head's width and serve all heads), rotation of the first ``rot``
     coordinates of every head by ``angles`` [nt, rot/2, 2], v <- (1 - mix) v + mix v_first,
     q written back in place, k and v stored at ``dest`` into the cache layer. ``v_keep``
     receives the values before mixing. The cache's value rows may be wider than the values
-    (vcache [pages, nkv, dvs, PAGE], dvs >= value_dim): the rest of a token's column is zeroed."""
+    (vcache [pages, nkv, dvs, PAGE], dvs >= value_dim): the rest of a token's column is zeroed.
+    ``k_inplace`` (no ``dest``): the keys are written back into their rows as the queries are."""
     _dev(qkv, "qkv", contiguous=False)
     nt, stride = _rows2d(qkv, "qkv")
     nq, nk, nv = num_heads * key_dim, num_kv_heads * key_dim, num_kv_heads * value_dim
@@ -992,8 +995,12 @@ def qk_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_dim: in
     normed = q_weight is not None
     if normed:
         _dev(q_weight, "q_weight", torch.float32); _dev(k_weight, "k_weight", torch.float32)
-        if q_weight.shape != (nq,) or k_weight.shape != (nk,):
-            raise KernelError("qk_prepare: norm weights must cover the whole q and k projections")
+        want = ((key_dim,), (key_dim,)) if per_head else ((nq,), (nk,))
+        if (tuple(q_weight.shape), tuple(k_weight.shape)) != want:
+            raise KernelError(f"qk_prepare: norm weights are {tuple(q_weight.shape)} / {tuple(k_weight.shape)}, "
+                              f"expected {want[0]} / {want[1]}")
+    if k_inplace and dest is not None:
+        raise KernelError("qk_prepare: the keys go back in place or to the cache, not both")
     if rot:
         _dev(angles, "angles", torch.float32)
         if tuple(angles.shape) != (nt, rot // 2, 2):
@@ -1020,10 +1027,10 @@ def qk_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_dim: in
             raise KernelError("qk_prepare: dest must hold one entry per token")
     _check(library().ta_qk_prepare(
         _stream(), c_int(_code(qkv.dtype)), _ptr(qkv), c_int(stride), _ptr(q_weight), _ptr(k_weight),
-        c_float(eps), c_int(int(normed)), _ptr(angles), c_int(rot), _ptr(mix), _ptr(v_first), _ptr(v_keep),
+        c_float(eps), c_int(2 if normed and per_head else int(normed)), _ptr(angles), c_int(rot), _ptr(mix), _ptr(v_first), _ptr(v_keep),
         _ptr(dest), _ptr(kcache if dest is not None else None), _ptr(vcache if dest is not None else None),
         c_int(nt), c_int(num_heads), c_int(num_kv_heads), c_int(key_dim), c_int(value_dim),
-        c_int(store_dim if dest is not None else value_dim)))
+        c_int(store_dim if dest is not None else value_dim), c_int(int(k_inplace))))
     return qkv
 
 
@@ -1332,22 +1339,97 @@ def wkv_recurrent(rkvg: torch.Tensor, low: torch.Tensor, heads: int, key_dim: in
     return o_out
 
 
-def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, heads: int, value_dim: int, weight: torch.Tensor,
-                   eps: float, out: torch.Tensor) -> torch.Tensor:
-    """out = rms_norm(o per head) * weight * silu(gate): o [parts, nt, H, dv] float32 planes that
-    add up, gate [nt, H*dv] (contiguous rows), weight [dv] for all heads or [H*dv]."""
+_GATE_ACTS = {"silu": 0, "sigmoid": 1}
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, heads: int, value_dim: int,
+                   weight: Optional[torch.Tensor], eps: float, out: torch.Tensor,
+                   gate_act: str = "silu") -> torch.Tensor:
+    """out = rms_norm(o per head) * weight * act(gate): o [parts, nt, H, dv] float32 planes that
+    add up, gate [nt, H*dv] (contiguous rows), weight [dv] for all heads, [H*dv], or None (the
+    plain division by the root mean square); act "silu" or "sigmoid". A norm over all heads at
+    once is the call with heads = 1 and value_dim = the whole row."""
     _dev(o, "o", torch.float32); _dev(gate, "gate", contiguous=False); _dev(out, "out", gate.dtype)
-    _dev(weight, "weight", torch.float32)
+    if weight is not None:
+        _dev(weight, "weight", torch.float32)
     nt, gs = _rows2d(gate, "gate")
     H, dv = heads, value_dim
+    if gate_act not in _GATE_ACTS:
+        raise KernelError(f"head_norm_gate: unknown gate activation {gate_act!r}")
     if o.dim() != 4 or o.shape[1:] != (nt, H, dv) or out.shape != (nt, H * dv) or gate.shape[1] != H * dv \
-            or weight.numel() not in (dv, H * dv):
+            or (weight is not None and weight.numel() not in (dv, H * dv)):
         raise KernelError(f"head_norm_gate: o {tuple(o.shape)} gate {tuple(gate.shape)} out {tuple(out.shape)} "
-                          f"weight {tuple(weight.shape)}")
-    _check(library().ta_gla_out_w(_stream(), c_int(_code(gate.dtype)), _ptr(o), c_int(o.shape[0]), _ptr(gate),
-                                  c_int(gs), c_longlong(0), _ptr(weight),
-                                  c_int(dv if weight.numel() == H * dv and H > 1 else 0), c_float(eps), c_int(nt),
-                                  c_int(H), c_int(dv), _ptr(out)))
+                          f"weight {None if weight is None else tuple(weight.shape)}")
+    wstride = dv if weight is not None and weight.numel() == H * dv and H > 1 else 0
+    _check(library().ta_gla_out_act(_stream(), c_int(_code(gate.dtype)), _ptr(o), c_int(o.shape[0]), _ptr(gate),
+                                    c_int(gs), c_longlong(0), _ptr(weight), c_int(wstride), c_float(eps),
+                                    c_int(nt), c_int(H), c_int(dv), c_int(_GATE_ACTS[gate_act]), _ptr(out)))
+    return out
+
+
+def decay_recurrent(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads: int, key_dim: int,
+                    value_dim: int, decays: torch.Tensor, q_scale: float, state: torch.Tensor, cu_q, slots,
+                    o_out: torch.Tensor) -> torch.Tensor:
+    """Linear attention with ONE fixed decay per head along every sequence: S <- decay_h S + k
+    v^T, o = S^T (q_scale * q). q, k, v sit at columns q_off, k_off, v_off of the rows of
+    ``proj`` (heads x key_dim, heads x key_dim, heads x value_dim). decays [H] float32 on the
+    device; ``state`` [slots, H, dk, dv] float32; o_out [gla_row_parts(dk), nt, H, dv] float32
+    planes that add up to the readout."""
+    _dev(proj, "proj", contiguous=False)
+    nt, stride = _rows2d(proj, "proj")
+    H, dk, dv = heads, key_dim, value_dim
+    batch = _step_tables(cu_q, slots, nt, "decay_recurrent")
+    _dev(decays, "decays", torch.float32); _dev(state, "state", torch.float32); _dev(o_out, "o_out", torch.float32)
+    ends = (q_off + H * dk, k_off + H * dk, v_off + H * dv)
+    if min(q_off, k_off, v_off) < 0 or max(ends) > proj.shape[1] or decays.shape != (H,) or state.dim() != 4 \
+            or state.shape[1:] != (H, dk, dv) or o_out.shape != (gla_row_parts(dk), nt, H, dv):
+        raise KernelError(f"decay_recurrent: shapes do not fit {H} heads of {dk} / {dv}: proj {tuple(proj.shape)} "
+                          f"offsets {(q_off, k_off, v_off)} decays {tuple(decays.shape)} state {tuple(state.shape)} "
+                          f"o_out {tuple(o_out.shape)}")
+    _check(library().ta_decay_recurrent(
+        _stream(), c_int(_code(proj.dtype)), _ptr(proj), c_int(stride), c_int(q_off), c_int(k_off), c_int(v_off),
+        _ptr(decays), c_float(q_scale), _ptr(state), _ptr(cu_q), _ptr(slots), c_int(batch), c_int(nt), c_int(H),
+        c_int(dk), c_int(dv), _ptr(o_out)))
+    return o_out
+
+
+def glu_limit(gate_up: torch.Tensor, out: torch.Tensor, limit: float, slope: float = 1.702,
+              shift: float = 1.0) -> torch.Tensor:
+    """Rows [gate | up] -> out = g * sigmoid(slope * g) * (u + shift) with g = min(gate, limit),
+    u = clamp(up, -limit, limit); float32 inside. gate_up [nt, 2n], out [nt, n] contiguous."""
+    _dev(gate_up, "gate_up", contiguous=False); _dev(out, "out", gate_up.dtype)
+    nt, ld = _rows2d(gate_up, "gate_up")
+    if gate_up.shape[1] % 2 or out.shape != (nt, gate_up.shape[1] // 2):
+        raise KernelError(f"glu_limit: gate_up {tuple(gate_up.shape)} / out {tuple(out.shape)}")
+    _check(library().ta_glu_limit(_stream(), c_int(_code(gate_up.dtype)), _ptr(gate_up), c_int(ld), _ptr(out),
+                                  c_int(nt), c_int(out.shape[1]), c_float(limit), c_float(slope), c_float(shift)))
+    return out
+
+
+def normed_mean(deltas: Sequence[torch.Tensor], weights: Sequence[torch.Tensor], eps: float,
+                out: torch.Tensor) -> torch.Tensor:
+    """out = mean over i of rms_norm(deltas[i], eps) * weights[i]: deltas float32 [nt, d] or
+    [planes, nt, d] (planes added in order), weights float32 [d], out float32 [nt, d]."""
+    _dev(out, "out", torch.float32)
+    nt, d = out.shape
+    n = len(deltas)
+    if not 1 <= n <= 4 or len(weights) != n:
+        raise KernelError(f"normed_mean: {n} branches with {len(weights)} weights (1 to 4 are taken)")
+    planes, plane = [], []
+    for i, (t, w) in enumerate(zip(deltas, weights)):
+        _dev(t, f"deltas[{i}]", torch.float32); _dev(w, f"weights[{i}]", torch.float32)
+        if t.dim() == 3 and t.shape[1:] == out.shape:
+            planes.append(t.shape[0]); plane.append(nt * d)
+        elif t.shape == out.shape:
+            planes.append(1); plane.append(0)
+        else:
+            raise KernelError(f"normed_mean: deltas[{i}] is {tuple(t.shape)}, out {tuple(out.shape)}")
+        if w.shape != (d,):
+            raise KernelError(f"normed_mean: weights[{i}] is {tuple(w.shape)}, expected {(d,)}")
+    dp = (c_void_p * n)(*[t.data_ptr() for t in deltas])
+    wp = (c_void_p * n)(*[w.data_ptr() for w in weights])
+    _check(library().ta_normed_mean(_stream(), c_int(n), dp, (c_int * n)(*planes), (c_longlong * n)(*plane), wp,
+                                    c_float(eps), _ptr(out), c_int(nt), c_int(d)))
     return out
 
 
@@ -1481,16 +1563,23 @@ def moe_max_rows(pairs: int, experts: int) -> int:
 
 
 def moe_route(logits: torch.Tensor, experts: int, top: int, chosen: torch.Tensor, weight: torch.Tensor,
-              score: str = "sigmoid", renormalize: bool = False):
+              score: str = "sigmoid", renormalize: bool = False, bias: Optional[torch.Tensor] = None):
     """chosen [nt, top] int32, weight [nt, top] float32: the ``top`` largest scores of the
-    first ``experts`` columns of logits [nt, >= experts] float32 (lowest index among equals)."""
+    first ``experts`` columns of logits [nt, >= experts] float32 (lowest index among equals).
+    bias [experts] float32: added to the logits first. "softmax" with ``renormalize`` is the
+    softmax over the chosen logits alone."""
     _dev(logits, "logits", torch.float32, contiguous=False)
     nt, ld = _rows2d(logits, "logits")
     _dev(chosen, "chosen", torch.int32); _dev(weight, "weight", torch.float32)
     if score not in _ROUTE_MODES or logits.shape[1] < experts or chosen.shape != (nt, top) or weight.shape != (nt, top):
         raise KernelError(f"moe_route: logits {tuple(logits.shape)} chosen {tuple(chosen.shape)} score {score!r}")
-    _check(library().ta_moe_route(_stream(), _ptr(logits), c_int(ld), c_int(nt), c_int(experts), c_int(top),
-                                  c_int(_ROUTE_MODES[score]), c_int(int(renormalize)), _ptr(chosen), _ptr(weight)))
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.shape != (experts,):
+            raise KernelError(f"moe_route: bias is {tuple(bias.shape)}, expected {(experts,)}")
+    _check(library().ta_moe_route_bias(_stream(), _ptr(logits), _ptr(bias), c_int(ld), c_int(nt), c_int(experts),
+                                       c_int(top), c_int(_ROUTE_MODES[score]), c_int(int(renormalize)),
+                                       _ptr(chosen), _ptr(weight)))
     return chosen, weight
 
 
@@ -1541,9 +1630,11 @@ def moe_gemm(a: torch.Tensor, w: torch.Tensor, tile_expert: torch.Tensor, out: t
 
 
 def moe_combine(rows: torch.Tensor, top: int, pair_row: torch.Tensor, weight, shared, shared_gate,
-                delta: torch.Tensor) -> torch.Tensor:
+                delta: torch.Tensor, extra: Optional[torch.Tensor] = None) -> torch.Tensor:
     """delta[t] = sum over the token's pairs of rows[pair_row] (* weight) + sigmoid(shared_gate[t,
-    0]) * shared[t]; shared [nt, d] or [planes, nt, d] float32; shared_gate float32 [nt, >= 1]."""
+    0]) * shared[t] (+ extra[t]); shared and extra [nt, d] or [planes, nt, d] float32;
+    shared_gate float32 [nt, >= 1]. ``extra``: what another sublayer adds to the stream beside
+    this one."""
     _dev(rows, "rows", torch.float32); _dev(pair_row, "pair_row", torch.int32); _dev(delta, "delta", torch.float32)
     nt, d = delta.shape
     if rows.shape[1] != d or pair_row.numel() != nt * top:
@@ -1562,7 +1653,17 @@ def moe_combine(rows: torch.Tensor, top: int, pair_row: torch.Tensor, weight, sh
         ng, gl = _rows2d(shared_gate, "shared_gate")
         if ng != nt:
             raise KernelError(f"moe_combine: shared_gate is {tuple(shared_gate.shape)}")
-    _check(library().ta_moe_combine(_stream(), _ptr(rows), c_int(d), c_int(top), _ptr(pair_row), _ptr(weight),
-                                    _ptr(shared), c_int(planes), c_longlong(plane), _ptr(shared_gate), c_int(gl),
-                                    _ptr(delta), c_int(nt)))
+    xplanes, xplane = 0, 0
+    if extra is not None:
+        _dev(extra, "extra", torch.float32)
+        if extra.dim() == 3 and extra.shape[1:] == delta.shape:
+            xplanes, xplane = extra.shape[0], nt * d
+        elif extra.shape == delta.shape:
+            xplanes = 1
+        else:
+            raise KernelError(f"moe_combine: extra is {tuple(extra.shape)}")
+    _check(library().ta_moe_combine_extra(_stream(), _ptr(rows), c_int(d), c_int(top), _ptr(pair_row), _ptr(weight),
+                                          _ptr(shared), c_int(planes), c_longlong(plane), _ptr(shared_gate),
+                                          c_int(gl), _ptr(extra), c_int(xplanes), c_longlong(xplane), _ptr(delta),
+                                          c_int(nt)))
     return delta

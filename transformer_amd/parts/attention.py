@@ -158,19 +158,21 @@ class NormedAttention(Part):
         self.spec, self.dtype = s, dtype
         self.nq, self.nkv, self.dk, self.dv = s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim
         self.width = (self.nq + self.nkv) * self.dk + self.nkv * self.dv
+        self.per_head = bool(getattr(s, "qk_norm_per_head", False))
         self.rotary = None
         if s.rot_dims:
             from ..config.spec import PositionSpec
-            self.rotary = build_part(PositionSpec(head_dim=s.rot_dims, theta=s.rot_base, style="half"),
-                                     dtype, device)
+            self.rotary = build_part(PositionSpec(head_dim=s.rot_dims, theta=s.rot_base, style="half",
+                                                  scaling=getattr(s, "rot_scaling", None)), dtype, device)
 
     def params(self):
         s = self.spec
         p = {"qkv.weight": Param((self.width, s.hidden), "matrix"),
              "out.weight": Param((s.hidden, self.nq * self.dv), "matrix")}
         if s.qk_norm:
-            p["q_norm.weight"] = Param((self.nq * self.dk,), "vector", init="around_one")
-            p["k_norm.weight"] = Param((self.nkv * self.dk,), "vector", init="around_one")
+            # one weight per coordinate of the projection, or (per head) one of the head's width
+            p["q_norm.weight"] = Param((self.dk if self.per_head else self.nq * self.dk,), "vector", init="around_one")
+            p["k_norm.weight"] = Param((self.dk if self.per_head else self.nkv * self.dk,), "vector", init="around_one")
         if s.value_mix is not None:
             p["value_mix"] = Param((), "vector", init="zero")    # a source holds it too, unused
         return p
@@ -220,7 +222,8 @@ class NormedAttention(Part):
         angles = self.rotary.angles(ctx) if self.rotary is not None else None
         kernels.qk_prepare(qkv, self.nq, self.nkv, self.dk, self.dv, float(s.eps),
                            self.w.get("q_norm.weight"), self.w.get("k_norm.weight"), angles, s.rot_dims,
-                           mix, first, keep, meta.dest if writes_cache else None, kc, vc)
+                           mix, first, keep, meta.dest if writes_cache else None, kc, vc,
+                           per_head=self.per_head)
         if not self._on_matrix_cores():
             o = ctx.ws.take("attention.o", (nt, self.nq * self.dv), self.dtype)
             kernels.attention_generic_dv(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,

@@ -206,3 +206,61 @@ class GatedPreNormBlock(Part):
 
 
 register_part("gated_prenorm", GatedPreNormBlock)
+
+
+class ParallelBlock(Part):
+    """h = norm1(x); x += mixer(h) + ffn(h): one norm, and both sublayers read its rows
+    (``ParallelBlockSpec``). The sum travels to the next norm as one pending delta: a
+    feed-forward that offers ``adds_extra`` takes the mixer's delta into its own last kernel;
+    for any other the two are laid side by side as planes, which the norm adds in order."""
+    folds_norms = False
+
+    def __init__(self, spec, dtype, device):
+        self.dtype = dtype
+        self.norm1 = build_part(spec.norm1, dtype, device)
+        self.mixer = build_part(spec.mixer, dtype, device)
+        self.ffn = build_part(spec.ffn, dtype, device) if spec.ffn is not None else None
+
+    def children(self):
+        c = {"norm1": self.norm1, "mixer": self.mixer}
+        if self.ffn is not None:
+            c["ffn"] = self.ffn
+        return c
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def step_planner(self):
+        f = getattr(self.mixer, "step_planner", None)
+        return f() if f is not None else None
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", False) for p in self.children().values())
+
+    def run(self, x, pending, ctx, cache, layer, writes_cache=True, after=None):
+        if not isinstance(pending, tuple):
+            raise ValueError("a parallel block takes a pending (delta, bias) pair from the block in front")
+        h = ctx.ws.take("block.h", x.shape, self.dtype)
+        with span(ctx, "norm"):
+            self.norm1.run(x, h, pending[0], pending[1])
+        with span(ctx, "mixer"):
+            delta, bias = self.mixer.run(h, ctx, cache, layer, writes_cache)
+        if self.ffn is None:
+            return delta, bias
+        with span(ctx, "ffn"):
+            if getattr(self.ffn, "adds_extra", False):
+                fd, fb = self.ffn.run(h, ctx, extra=delta)
+            else:
+                fd, fb = self.ffn.run(h, ctx)
+                planes = [t for d in (delta, fd) for t in (d if d.dim() == 3 else d.unsqueeze(0))]
+                both = ctx.ws.take("block.sum", (len(planes), *x.shape), torch.float32)
+                for i, t in enumerate(planes):
+                    both[i].copy_(t)
+                fd = both
+        if bias is not None and fb is not None:
+            raise ValueError("a parallel block carries one pending bias row, and both sublayers left one")
+        return fd, bias if bias is not None else fb
+
+
+register_part("parallel_prenorm", ParallelBlock)

@@ -125,12 +125,20 @@ class RoutedMLP(Part):
     routing; the experts' products walk that list tile by tile, each tile with its expert's
     matrix; the rows go back to their tokens in float32."""
     graph_safe = True
+    adds_extra = True       # ``run(..., extra=)``: the last kernel also adds another sublayer's delta
 
     def __init__(self, spec, dtype, device):
         s = spec
         if not 1 <= s.top <= s.experts or s.intermediate < 1:
             raise PartError(f"routed feed-forward: top {s.top} of {s.experts} experts of {s.intermediate}")
-        if s.activation not in kernels._MOE_ACTS or s.activation not in kernels._ACTIVATIONS:
+        form = getattr(s, "form", "mlp")
+        if form not in ("mlp", "limited_glu"):
+            raise PartError(f"routed feed-forward: unknown form {form!r}")
+        self.limited = form == "limited_glu"
+        if self.limited:
+            if not s.limit > 0 or (s.shared_intermediate is not None and not s.shared_limit > 0):
+                raise PartError(f"routed feed-forward: limits must be positive, got {s.limit} / {s.shared_limit}")
+        elif s.activation not in kernels._MOE_ACTS or s.activation not in kernels._ACTIVATIONS:
             raise PartError(f"unknown expert activation {s.activation!r}")
         if s.score not in ("sigmoid", "softmax") or s.weight_on not in ("input", "output"):
             raise PartError(f"routed feed-forward: score {s.score!r}, weight on {s.weight_on!r}")
@@ -139,22 +147,43 @@ class RoutedMLP(Part):
 
     def params(self):
         s = self.spec
+        # limited_glu: an expert's first matrix is [gate rows | up rows]
+        first, k = ("gate_up", 2) if self.limited else ("up", 1)
         p = {"router.weight": Param((s.experts + int(self.gated_shared), s.hidden), "matrix"),
-             "experts.up.weight": Param((s.experts * s.intermediate, s.hidden), "matrix"),
+             f"experts.{first}.weight": Param((s.experts * k * s.intermediate, s.hidden), "matrix"),
              "experts.down.weight": Param((s.experts * s.hidden, s.intermediate), "matrix")}
+        if getattr(s, "router_bias", False):
+            p["router.bias"] = Param((s.experts,), "vector")
         if s.shared_intermediate is not None:
-            p["shared.up.weight"] = Param((s.shared_intermediate, s.hidden), "matrix")
+            p[f"shared.{first}.weight"] = Param((k * s.shared_intermediate, s.hidden), "matrix")
             p["shared.down.weight"] = Param((s.hidden, s.shared_intermediate), "matrix")
         return p
 
-    def run(self, h, ctx):
+    def _first(self, a, w, tile_expert, ws, name, n, act_limit):
+        """The first product of the experts (tile_expert given) or of the shared expert with
+        its activation: rows [.., n] in the engine's type."""
+        s, rows = self.spec, a.shape[0]
+        k = 2 if self.limited else 1
+        pre = ws.take(name + ".pre", (rows, k * n), self.dtype)
+        if tile_expert is not None:
+            kernels.moe_gemm(a, w, tile_expert, pre, None if self.limited else s.activation)
+        else:
+            linear(a, w, pre)
+        if not self.limited:
+            if tile_expert is None:
+                kernels.activation(pre, pre, s.activation)
+            return pre
+        return kernels.glu_limit(pre, ws.take(name, (rows, n), self.dtype), float(act_limit),
+                                 float(s.gate_slope), float(s.up_shift))
+
+    def run(self, h, ctx, extra=None):
         s, nt, d = self.spec, h.shape[0], self.spec.hidden
         E, top, ff = s.experts, s.top, s.intermediate
         ws = ctx.ws
         logits = linear(h, self.w["router.weight"], ws.take("moe.logits", (nt, E + int(self.gated_shared)), torch.float32))
         chosen = ws.take("moe.chosen", (nt, top), torch.int32)
         weight = ws.take("moe.weight", (nt, top), torch.float32)
-        kernels.moe_route(logits, E, top, chosen, weight, s.score, s.renormalize)
+        kernels.moe_route(logits, E, top, chosen, weight, s.score, s.renormalize, bias=self.w.get("router.bias"))
         if getattr(ctx, "dump", None) is not None:
             ctx.dump("experts", chosen)
         rows = kernels.moe_max_rows(nt * top, E)
@@ -164,20 +193,21 @@ class RoutedMLP(Part):
         kernels.moe_plan(chosen, E, row_pair, tile_expert, pair_row)
         on_input = s.weight_on == "input"
         a = kernels.moe_gather(h, top, row_pair, weight if on_input else None, ws.take("moe.a", (rows, d), self.dtype))
-        up = self.w["experts.up.weight"].view(E, ff, d)
+        first, k = ("gate_up", 2) if self.limited else ("up", 1)
+        up = self.w[f"experts.{first}.weight"].view(E, k * ff, d)
         down = self.w["experts.down.weight"].view(E, d, ff)
         if up.dtype != self.dtype:
             raise PartError(f"the experts' matrices are {up.dtype}, the engine computes in {self.dtype}")
-        mid = kernels.moe_gemm(a, up, tile_expert, ws.take("moe.mid", (rows, ff), self.dtype), s.activation)
+        mid = self._first(a, up, tile_expert, ws, "moe.mid", ff, getattr(s, "limit", 0.0))
         out = kernels.moe_gemm(mid, down, tile_expert, ws.take("moe.out", (rows, d), torch.float32))
         shared = None
         if s.shared_intermediate is not None:
-            u = linear(h, self.w["shared.up.weight"], ws.take("moe.shared_up", (nt, s.shared_intermediate), self.dtype))
-            kernels.activation(u, u, s.activation)
+            u = self._first(h, self.w[f"shared.{first}.weight"], None, ws, "moe.shared_up", s.shared_intermediate,
+                            getattr(s, "shared_limit", 0.0))
             shared = linear_delta(u, self.w["shared.down.weight"], ws, "moe.shared")
         delta = kernels.moe_combine(out, top, pair_row, None if on_input else weight, shared,
                                     logits[:, E:] if self.gated_shared else None,
-                                    ws.take("moe.delta", (nt, d), torch.float32))
+                                    ws.take("moe.delta", (nt, d), torch.float32), extra=extra)
         return delta, None
 
 

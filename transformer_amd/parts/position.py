@@ -20,6 +20,24 @@ from .. import kernels
 from .base import Part, PartError, register_part
 
 
+def scaled_frequencies(dims: int, base: float, scaling=None) -> np.ndarray:
+    """f_j = base^(-2j/dims), j < dims/2, float64. scaling (factor, low, high, original) slows
+    the long wavelengths l = 2 pi / f: f / factor where l > original/low, f where l <
+    original/high, and between the two (1 - s) f / factor + s f with s = (original/l - low) /
+    (high - low)."""
+    j = np.arange(dims // 2, dtype=np.float64)
+    f = float(base) ** (-2.0 * j / dims)
+    if scaling is None:
+        return f
+    factor, low, high, original = (float(v) for v in scaling)
+    if not (factor > 0 and original > 0 and high > low >= 0):
+        raise PartError(f"rotary scaling: factor {factor}, low {low}, high {high}, original {original}")
+    wavelength = 2.0 * np.pi / f
+    share = np.clip((original / wavelength - low) / (high - low), 0.0, 1.0)
+    blended = (1.0 - share) * f / factor + share * f
+    return np.where(wavelength < original / high, f, np.where(wavelength > original / low, f / factor, blended))
+
+
 class Rotary(Part):
     graph_safe = True
 
@@ -30,17 +48,17 @@ class Rotary(Part):
             raise PartError(f"unknown rotary pairing {spec.style!r}")
         self.head_dim = spec.head_dim
         self.interleaved = spec.style == "interleaved"
-        j = np.arange(spec.head_dim // 2, dtype=np.float64)
-        inv = float(spec.theta) ** (-2.0 * j / spec.head_dim)
+        inv = scaled_frequencies(spec.head_dim, float(spec.theta), getattr(spec, "scaling", None))
         self.inv_freq = torch.tensor(inv.astype(np.float32), device=device)
-        self.key = ("rope", spec.head_dim, float(spec.theta))
+        scaling = getattr(spec, "scaling", None)
+        self.key = ("rope", spec.head_dim, float(spec.theta), None if scaling is None else tuple(scaling))
 
     def angles(self, ctx):
         """(cos, sin) of every token of the step, computed once per step and shared
         by all layers that rotate with the same frequencies."""
         table = ctx.shared.get(self.key)
         if table is None:
-            out = ctx.ws.take(f"rope.angles.{self.head_dim}.{self.key[2]}",
+            out = ctx.ws.take("rope.angles." + ".".join(str(k) for k in self.key[1:]),
                               (ctx.nt, self.head_dim // 2, 2), torch.float32)
             table = kernels.rope_table(ctx.positions, self.inv_freq, out)
             ctx.shared[self.key] = table

@@ -158,6 +158,84 @@ class BonusRecurrence(Part):
         return linear_delta(g, self.w["out.weight"], ctx.ws, "bonus.delta"), None
 
 
+class DecayLinearAttention(Part):
+    """Linear attention with one fixed decay per head and no softmax or denominator
+    (``DecayLinearAttentionSpec``): S_t = decay_h S_{t-1} + k_t v_t^T, o_t = S_t^T q_t.
+
+    One merged product gives [q | k | v | gate]. Options of the spec, each a kernel step of its
+    own: an activation on q, k, v; a rotation of the first coordinates of every head of q and k
+    (the keys go back into their rows); a scale on the keys, which the recurrence applies to
+    the queries instead (the readout is linear in both); the norm of the readout per head or
+    over all heads at once, with or without a weight; the gate's activation. The recurrence is
+    the kernel of ``GatedLinearAttention`` with the head's constant in place of a decay per
+    key channel and token: state, decays and readout stay float32, tokens are walked in order,
+    so a cut of the sequence changes nothing."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        s = spec
+        if min(s.num_heads, s.key_dim, s.value_dim) < 1:
+            raise PartError(f"linear attention: {s.num_heads} heads of {s.key_dim} / {s.value_dim}")
+        if len(s.decays) != s.num_heads:
+            raise PartError(f"linear attention: {len(s.decays)} decays for {s.num_heads} heads")
+        if any(not 0.0 <= float(a) <= 1.0 for a in s.decays):
+            raise PartError(f"linear attention: decays must lie in [0, 1], got {tuple(s.decays)}")
+        if s.input_activation not in (None, "silu") or s.gate_activation not in ("silu", "sigmoid"):
+            raise PartError(f"linear attention: activations {s.input_activation!r} / {s.gate_activation!r}")
+        if s.head_norm not in ("per_head", "all_heads"):
+            raise PartError(f"linear attention: unknown head_norm {s.head_norm!r}")
+        if s.rot_dims % 2 or not 0 <= s.rot_dims <= s.key_dim:
+            raise PartError(f"{s.rot_dims} rotated coordinates do not fit heads of {s.key_dim}")
+        self.spec, self.dtype = s, dtype
+        self.nk, self.nv = s.num_heads * s.key_dim, s.num_heads * s.value_dim
+        self.width = 2 * self.nk + 2 * self.nv
+        self.decays = torch.tensor([float(a) for a in s.decays], dtype=torch.float32, device=device)
+        self.rotary = None
+        if s.rot_dims:
+            from ..config.spec import PositionSpec
+            from .base import build_part
+            self.rotary = build_part(PositionSpec(head_dim=s.rot_dims, theta=s.rot_base, style="half",
+                                                  scaling=s.rot_scaling), dtype, device)
+
+    def params(self):
+        s = self.spec
+        p = {"in.weight": Param((self.width, s.hidden), "matrix"),       # q, k, v, gate
+             "out.weight": Param((s.hidden, self.nv), "matrix")}
+        if s.norm_weight:
+            n = self.nv if s.head_norm == "all_heads" else s.value_dim
+            p["norm.weight"] = Param((n,), "vector", init="around_one")
+        return p
+
+    def cache_need(self):
+        s = self.spec
+        return StateNeed((s.num_heads, s.key_dim, s.value_dim), torch.float32)
+
+    def run(self, h, ctx, cache, layer, writes_cache=True):
+        s, nt = self.spec, h.shape[0]
+        H, dk, dv = s.num_heads, s.key_dim, s.value_dim
+        proj = linear(h, self.w["in.weight"], ctx.ws.take("decay_attention.in", (nt, self.width), self.dtype))
+        qkv = proj[:, :2 * self.nk + self.nv]
+        if s.input_activation is not None:
+            kernels.activation(qkv, qkv, s.input_activation)
+        if self.rotary is not None:
+            kernels.qk_prepare(qkv, H, H, dk, dv, float(s.eps), None, None, self.rotary.angles(ctx), s.rot_dims,
+                               k_inplace=True)
+        o = kernels.decay_recurrent(proj, 0, self.nk, 2 * self.nk, H, dk, dv, self.decays, float(s.key_scale),
+                                    cache.layer_state(layer), ctx.cu_q, ctx.slots,
+                                    ctx.ws.take("decay_attention.o", (kernels.gla_row_parts(dk), nt, H, dv),
+                                                torch.float32))
+        gate = proj[:, 2 * self.nk + self.nv:]
+        gated = ctx.ws.take("decay_attention.gated", (nt, self.nv), self.dtype)
+        if s.head_norm == "all_heads":
+            kernels.head_norm_gate(o.view(o.shape[0], nt, 1, self.nv), gate, 1, self.nv, self.w.get("norm.weight"),
+                                   float(s.eps), gated, s.gate_activation)
+        else:
+            kernels.head_norm_gate(o, gate, H, dv, self.w.get("norm.weight"), float(s.eps), gated,
+                                   s.gate_activation)
+        return linear_delta(gated, self.w["out.weight"], ctx.ws, "decay_attention.delta"), None
+
+
 register_part("diagonal_recurrence", DiagonalRecurrence)
+register_part("decay_linear_attention", DecayLinearAttention)
 register_part("bonus_recurrence", BonusRecurrence)
 register_part("gated_linear_attention", GatedLinearAttention)
