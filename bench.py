@@ -213,9 +213,62 @@ def kunitar_shapes():
             "w4096": shape(4096, 32, 1536, 512, 4096, 14336, 64, 64, 6, 1408, 2816, 32000)}
 
 
+def luduvik_shapes():
+    """Layer sizes that resemble real models' (random weights): Luduvik models whose layers are
+    all lightning or all parallel (each with the routed feed-forward), the mixed order, and the
+    closest layers of the other decoders at the same width and heads: the Vametar decoder's gated
+    linear attention and its attention, the Kunitar decoder's recurrence with the routed
+    feed-forward of the same experts, and the Llama layer."""
+    def shape(width, heads, kv, lin_heads, experts, top, eff, sff, ff, vocab):
+        moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": eff, "limit": 7.0},
+               "shared": {"ff": sff, "limit": 7.0}}
+        decay = [1.0 - 2.0 ** -(5.0 + 4.0 * i / lin_heads) for i in range(lin_heads)]
+        light = {"type": "lightning", "mixer": {"heads": lin_heads, "dim": 128, "vdim": 128, "decay": decay}, "mlp": moe}
+        par = {"type": "parallel", "mlp": moe, "mixer": {
+            "left": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+            "right": {"heads": lin_heads, "dim": 128, "vdim": 128, "decay": decay, "rot": {"base": 10000.0, "dims": 128}}}}
+        base = {"architecture": "Luduvik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}}
+        kinds = {"lightning": [light] * 4, "parallel": [par] * 4, "mixed": [light, par, light, light]}
+        vam = {"architecture": "Vametar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
+               "logit_scale": 2.0, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}}
+        dense = {"kind": "dense", "ff": ff}
+        near = {
+            "vametar_gla": ("Vametar", {**vam, "layers": [{"type": "gla", "mlp": dense, "mixer": {
+                "heads": lin_heads, "dim": 128, "vdim": 128, "tau": 16.0, "rank": 16}}] * 4}),
+            "vametar_attention": ("Vametar", {**vam, "layers": [{"type": "attention", "mlp": dense, "mixer": {
+                "heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                "rot": {"base": 500000.0, "dims": 64}}}] * 4}),
+            "kunitar_wkv_moe": ("Kunitar", {"architecture": "Kunitar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+                                            "embedding": {"scale": 2.0}, "layers": [{
+                                                "type": "wkv", "mixer": {"heads": 2 * lin_heads, "dim": 64, "decay_rank": 64},
+                                                "mlp": {"kind": "moe", "router": {"experts": experts, "top": top},
+                                                        "expert": {"ff": eff}, "shared": {"ff": sff}}}] * 4}),
+            "llama": ("llama", {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": width,
+                                "num_attention_heads": heads, "num_key_value_heads": kv, "head_dim": 128,
+                                "intermediate_size": ff, "vocab_size": vocab, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+                                "tie_word_embeddings": False, "max_position_embeddings": 1 << 20, "rope_scaling": None,
+                                "num_hidden_layers": 4}),
+        }
+        return base, kinds, near
+    return {"w2048": shape(2048, 16, 4, 16, 32, 4, 1024, 2048, 8192, 32000),
+            "w4096": shape(4096, 32, 8, 32, 64, 6, 1408, 2816, 14336, 32000)}
+
+
 def _routed_parts(model):
     return [b.ffn for b in model.blocks if getattr(getattr(b, "ffn", None), "spec", None) is not None
             and getattr(b.ffn.spec, "kind", "") == "routed_mlp"]
+
+
+def _expert_entries(sp):
+    """Matrix entries of one routed expert: up and down, and a gate matrix where it has one."""
+    return (3 if getattr(sp, "form", "mlp") == "limited_glu" else 2) * sp.hidden * sp.intermediate
+
+
+def _leaf_mixers(m):
+    """The mixers of a block: itself, or the branches of mixers that run side by side."""
+    subs = getattr(m, "branches", None)
+    return [m] if subs is None else [x for b in subs for x in _leaf_mixers(b)]
 
 
 def generic_step_bytes(model, contexts):
@@ -242,8 +295,7 @@ def generic_step_bytes(model, contexts):
             per_seq += 2 * n * torch.empty((), dtype=need.dtype).element_size()
     for f in _routed_parts(model):       # of the experts only those that the step's tokens can reach
         sp = f.spec
-        one = 2 * sp.hidden * sp.intermediate * item
-        w -= max(0, sp.experts - len(contexts) * sp.top) * one
+        w -= max(0, sp.experts - len(contexts) * sp.top) * _expert_entries(sp) * item
     windowed = 0
     for need in model.cache_needs:       # a window bounds what a layer reads of a sequence
         if isinstance(need, KVNeed) and need.window is not None:
@@ -262,10 +314,9 @@ def generic_prefill_flops(model, T):
     mats -= sum(t.numel() for n, t in model.tensors.items() if n.endswith(".table"))
     for f in _routed_parts(model):       # a token goes through ``top`` of the experts
         sp = f.spec
-        mats -= (sp.experts - sp.top) * 2 * sp.hidden * sp.intermediate
+        mats -= (sp.experts - sp.top) * _expert_entries(sp)
     fl = 2 * T * mats + 2 * model.spec.hidden * model.spec.vocab
-    for blk in model.blocks:
-        m = blk.mixer
+    for m in (x for blk in model.blocks for x in _leaf_mixers(blk.mixer)):
         need = m.cache_need()
         if isinstance(need, KVNeed):
             window = getattr(m.spec, "window", None)
@@ -327,6 +378,42 @@ def bench_kunitar(a):
             else:
                 lay = (lay * (-(-layers // len(lay))))[:layers]
                 model = ta.random_model({**base, "layers": lay}, seed=0, dtype=a.dtype, architecture="Kunitar")
+            rows[name] = _design_row(model, a, dkey)
+            del model
+            torch.cuda.empty_cache()
+            print(f"[bench] {size} {name}: {rows[name]}", file=sys.stderr, flush=True)
+        out["sizes"][size] = rows
+    print(json.dumps(out))
+    return 0
+
+
+def bench_luduvik(a):
+    """Prefill and decode throughput of Luduvik models whose layers are all lightning, all
+    parallel, and the mixed order, beside the closest layers of the other decoders at the same
+    width. One JSON line of its own; the default workload is untouched."""
+    import torch
+    import transformer_amd as ta
+    dkey = "bf16" if a.dtype == "bfloat16" else "fp32"
+    layers = a.layers or 4
+    out = {"design": "luduvik", "dtype": dkey, "layers": layers, "batch": a.batch,
+           "prefill_tokens": a.prefill_tokens, "data": "synthetic", "sizes": {}}
+
+    def fit(lay):
+        return (list(lay) * (-(-layers // len(lay))))[:layers]
+
+    for size, (base, kinds, near) in luduvik_shapes().items():
+        if a.design_size and size not in a.design_size.split(","):
+            continue
+        cases = [(n, arch, c) for n, (arch, c) in near.items()] + \
+                [(n, "Luduvik", {**base, "layers": lay}) for n, lay in kinds.items()]
+        if a.design_case:
+            cases = [c for c in cases if c[0] in a.design_case.split(",")]
+        rows = {}
+        for name, arch, cfg in cases:
+            if arch == "llama":
+                model = ta.random_model(ta.LlamaConfig.from_dict({**cfg, "num_hidden_layers": layers}), seed=0, dtype=a.dtype)
+            else:
+                model = ta.random_model({**cfg, "layers": fit(cfg["layers"])}, seed=0, dtype=a.dtype, architecture=arch)
             rows[name] = _design_row(model, a, dkey)
             del model
             torch.cuda.empty_cache()
@@ -419,14 +506,16 @@ def main():
                     help="tokens of the prompt whose step is timed (the line's \"prefill\")")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
-    ap.add_argument("--design", default=None, choices=["vametar", "kunitar"],
+    ap.add_argument("--design", default=None, choices=["vametar", "kunitar", "luduvik"],
                     help="instead of the default workload: prefill and decode of this design at a few "
                          "layer sizes, beside the Llama decoder at the same sizes (a line of its own)")
     ap.add_argument("--design-size", default=None, help="with --design: only these sizes (w2048,w4096)")
-    ap.add_argument("--design-case", default=None, help="with --design kunitar: only these rows (llama,latent,...)")
+    ap.add_argument("--design-case", default=None, help="with --design kunitar or luduvik: only these rows (llama,latent,...)")
     a = ap.parse_args()
     if a.design == "kunitar" and a.gpus == 1:
         return bench_kunitar(a)
+    if a.design == "luduvik" and a.gpus == 1:
+        return bench_luduvik(a)
     if a.design and a.gpus == 1:
         return bench_design(a)
     if a.gpus != 1:
