@@ -97,6 +97,10 @@ CFG_D = {
 }
 CONFIGS = {"A": (CFG_A, 31), "B": (CFG_B, 32), "C": (CFG_C, 33), "D": (CFG_D, 34)}
 STORAGE = {"float32": "F32", "bfloat16": "BF16"}
+# a bfloat16 engine may choose another expert than the plain model where the two logits are this
+# close (the logits spread over several units; rounding of the rows in front of the router moves
+# them by up to a tenth)
+SLACK = 0.15
 # largest allowed rms(engine - plain) / rms(plain) over a row of logits
 TOL = {"float32": 2e-4, "bfloat16": 1e-1}
 
@@ -225,6 +229,6 @@ def check_against_plain(name, dtype, edit, toks, got, routes=None, what=""):
     if dtype == "float32" or not routes:
         want = plain_logits(name, dtype, edit, tuple(toks))
     else:
-        want = plain(name, dtype, edit).forward(list(toks), routes=routes)
+        want = plain(name, dtype, edit).forward(list(toks), routes=routes, slack=SLACK)
     err = row_error(got, want[:len(got)]).max()
     assert err < TOL[dtype], f"{what}: {err}"

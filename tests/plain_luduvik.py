@@ -202,7 +202,7 @@ def moe(h, w, p, m, forced=None, slack=0.0):
             if set(forced[t]) != set(chosen[t]):
                 assert len(set(forced[t])) == len(forced[t]), f"token {t}: an expert chosen twice"
                 assert z[t, forced[t]].min() >= z[t, chosen[t]].min() - slack, \
-                    f"token {t}: experts {forced[t]} chosen, {chosen[t]} have the largest logits"
+                    f"token {t}: experts {forced[t]} chosen, {chosen[t]} have the largest logits: {z[t]}"
         zc = np.take_along_axis(z, forced, axis=-1)
         e = np.exp(zc - zc.max(axis=-1, keepdims=True))
         chosen, weight = forced, e / e.sum(axis=-1, keepdims=True)

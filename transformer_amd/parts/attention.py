@@ -184,7 +184,7 @@ class NormedAttention(Part):
     # (float32, other widths) runs the vector-ALU kernel on values of their own width.
     def _on_matrix_cores(self) -> bool:
         return (self.dtype == torch.bfloat16 and self.dk % 32 == 0 and 32 <= self.dk <= 256
-                and self.dv <= self.dk)
+                and self.dv <= self.dk and self.width % 8 == 0)     # rows of [q | k | v] start on 16 bytes
 
     def cache_need(self):
         return KVNeed(self.nkv, self.dk, self.spec.window, self.dk if self._on_matrix_cores() else self.dv)
