@@ -81,6 +81,23 @@ def test_limited_gate(dtype, limit):
     _close(_np(out), g * P.sigmoid(g) * u, dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geom", [(3072, 4096, 0), (24, 40, 8), (24, 40, 4), (20, 36, 0), (6144, 8192, 2048)])
+def test_silu_in_place_on_the_first_columns_of_wider_rows(dtype, geom):
+    """q, k, v of the lightning mixer are activated in place inside the rows [q | k | v | gate];
+    rows that start on 16 bytes take the kernel with wide loads, the others the plain one."""
+    from transformer_amd import kernels
+    n, width, first = geom
+    rng = np.random.default_rng(n)
+    rows = _bf(3 * rng.standard_normal((5, width)), dtype)
+    t = _t(rows, TD[dtype])
+    kernels.activation(t[:, first:first + n], t[:, first:first + n], "silu")
+    want = rows.copy()
+    want[:, first:first + n] = P.silu(rows[:, first:first + n])
+    _close(_np(t), want, dtype)
+    assert np.array_equal(_np(t)[:, first + n:], rows[:, first + n:]) and np.array_equal(_np(t)[:, :first], rows[:, :first])
+
+
 @pytest.mark.parametrize("geom", [(5, 2), (3, 3), (1, 1), (16, 1), (9, 4), (64, 6)])
 def test_router_bias_and_softmax_over_the_chosen(geom):
     from transformer_amd import kernels

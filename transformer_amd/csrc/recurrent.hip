@@ -825,6 +825,49 @@ __global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o
   }
 }
 
+// The same for wide heads (all heads normed as one row of thousands of columns): four waves share
+// a row, each thread keeps its columns in registers.
+template <typename T>
+__global__ __launch_bounds__(256) void gla_out_wide_kernel(const float* __restrict__ o, int parts, size_t plane,
+                                                           const T* __restrict__ proj, int stride,
+                                                           const float* __restrict__ w, int wstride, float eps,
+                                                           int H, int dv, T* __restrict__ out, int gate_act) {
+  constexpr int PER = 16;                 // columns a thread can own: rows of up to 256 * PER
+  __shared__ float red[4];
+  const size_t t = blockIdx.x;
+  const int h = blockIdx.y;
+  const float* src = o + (t * H + h) * dv;
+  float v[PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    v[i] = c < dv ? src[c] : 0.f;
+  }
+  for (int p = 1; p < parts; ++p)
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      if (c < dv) v[i] += src[p * plane + c];
+    }
+#pragma unroll
+  for (int i = 0; i < PER; ++i) ss += v[i] * v[i];
+  ss = wave_sum(ss);
+  if (threadIdx.x % TA_WAVE == 0) red[threadIdx.x / TA_WAVE] = ss;
+  __syncthreads();
+  const float f = rsqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)dv + eps);
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < dv) {
+      const float g = to_f32(proj[t * stride + h * dv + c]);
+      const float sg = 1.0f / (1.0f + expf(-g));
+      const float wc = w ? w[h * wstride + c] : 1.0f;
+      out[t * (size_t)(H * dv) + h * dv + c] = from_f32<T>(v[i] * f * wc * (gate_act == 1 ? sg : g * sg));
+    }
+  }
+}
+
 // o: [parts, nt, H, dv] float32 planes that add up to the readout; the gate's pre-activation sits
 // at element goff of proj, ``stride`` elements between tokens; w [dv] shared by the heads
 // (wstride 0) or [H, dv] (wstride dv); out [nt, H*dv] = rms_norm(o per head) * w * silu(gate).
@@ -838,6 +881,13 @@ extern "C" int ta_gla_out_act(hipStream_t stream, int dtype, const float* o, int
   if (nt == 0) return 0;
   dim3 g(nt, H);
   const size_t plane = (size_t)nt * H * dv, lds = (size_t)dv * sizeof(float);
+  if (dv > 512 && dv <= 4096 && (dtype == TA_F32 || dtype == TA_BF16)) {
+    if (dtype == TA_F32)
+      gla_out_wide_kernel<float><<<g, 256, 0, stream>>>(o, parts, plane, (const float*)proj + goff, stride, w, wstride, eps, H, dv, (float*)out, gate_act);
+    else
+      gla_out_wide_kernel<bf16_t><<<g, 256, 0, stream>>>(o, parts, plane, (const bf16_t*)proj + goff, stride, w, wstride, eps, H, dv, (bf16_t*)out, gate_act);
+    return ta_check_launch("ta_gla_out");
+  }
   if (dtype == TA_F32)
     gla_out_kernel<float><<<g, 64, lds, stream>>>(o, parts, plane, (const float*)proj + goff, stride, 0, w, wstride, eps, H, dv, (float*)out, gate_act);
   else if (dtype == TA_BF16)

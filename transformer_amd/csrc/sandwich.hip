@@ -166,6 +166,28 @@ __global__ __launch_bounds__(256) void activation_kernel(const T* __restrict__ i
   }
 }
 
+// Rows whose starts and lengths are multiples of 16 bytes, no side table: a thread takes 16 bytes
+// of a row at a time.
+template <typename T>
+__global__ __launch_bounds__(256) void activation_vec_kernel(const T* __restrict__ in, int in_stride,
+                                                             T* __restrict__ out, int out_stride, int n, int act) {
+  constexpr int W = 16 / sizeof(T);
+  const size_t t = blockIdx.y;
+  for (int c = (blockIdx.x * 256 + threadIdx.x) * W; c < n; c += gridDim.x * 256 * W) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(in + t * in_stride + c);
+    T a[W];
+    __builtin_memcpy(a, &raw, 16);
+    float v[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) v[i] = act_apply(act, to_f32(a[i]));
+#pragma unroll
+    for (int i = 0; i < W; ++i) a[i] = from_f32<T>(v[i]);
+    uint4 res;
+    __builtin_memcpy(&res, a, 16);
+    *reinterpret_cast<uint4*>(out + t * out_stride + c) = res;
+  }
+}
+
 // out[t, c] = act(in[t, c]) (* side[t, c]); rows may be strided. side: float32 or null.
 extern "C" int ta_activation(hipStream_t stream, int dtype, int act, const void* in, int in_stride, void* out,
                              int out_stride, const float* side, int side_stride, int nt, int n) {
@@ -177,6 +199,20 @@ extern "C" int ta_activation(hipStream_t stream, int dtype, int act, const void*
     if (gx > 64) gx = 64;
     dim3 g(gx, rows);
     const float* sd = side ? side + (size_t)t0 * side_stride : nullptr;
+    const int W = dtype == TA_F32 ? 4 : 8;
+    if (!side && (dtype == TA_F32 || dtype == TA_BF16) && n % W == 0 && in_stride % W == 0 && out_stride % W == 0 &&
+        (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0) {
+      int vx = (n / W + 255) / 256;
+      if (vx > 16) vx = 16;
+      dim3 gv(vx, rows);
+      if (dtype == TA_F32)
+        activation_vec_kernel<float><<<gv, 256, 0, stream>>>((const float*)in + (size_t)t0 * in_stride, in_stride,
+                                                             (float*)out + (size_t)t0 * out_stride, out_stride, n, act);
+      else
+        activation_vec_kernel<bf16_t><<<gv, 256, 0, stream>>>((const bf16_t*)in + (size_t)t0 * in_stride, in_stride,
+                                                              (bf16_t*)out + (size_t)t0 * out_stride, out_stride, n, act);
+      continue;
+    }
     if (dtype == TA_F32)
       activation_kernel<float><<<g, 256, 0, stream>>>((const float*)in + (size_t)t0 * in_stride, in_stride,
                                                       (float*)out + (size_t)t0 * out_stride, out_stride, n, act, sd, side_stride);
@@ -226,6 +262,59 @@ __global__ __launch_bounds__(256) void normed_mean_kernel(MeanBranches br, int n
   }
 }
 
+// d % 4 == 0, d <= 4096, every plane and pointer a multiple of 16 bytes: a thread keeps its runs
+// of four columns of a branch and of the mean in registers, so every plane is read once and the
+// loads of one branch do not wait for one another.
+__global__ __launch_bounds__(256) void normed_mean_vec_kernel(MeanBranches br, int n, float eps,
+                                                              float* __restrict__ out, int d) {
+  __shared__ float red[4];
+  constexpr int VMAX = 4;
+  const size_t base = (size_t)blockIdx.x * d;
+  const float inv = 1.0f / (float)n;
+  float4 acc[VMAX];
+#pragma unroll
+  for (int i = 0; i < VMAX; ++i) acc[i] = float4{0.f, 0.f, 0.f, 0.f};
+  for (int k = 0; k < n; ++k) {
+    const MeanBranch b = br.b[k];
+    float4 v[VMAX], wv[VMAX];
+#pragma unroll
+    for (int i = 0; i < VMAX; ++i) {
+      const int c = 4 * (threadIdx.x + 256 * i);
+      if (c < d) {
+        v[i] = *reinterpret_cast<const float4*>(b.delta + base + c);
+        wv[i] = *reinterpret_cast<const float4*>(b.w + c);
+      } else {
+        v[i] = wv[i] = float4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    for (int p = 1; p < b.planes; ++p)
+#pragma unroll
+      for (int i = 0; i < VMAX; ++i) {
+        const int c = 4 * (threadIdx.x + 256 * i);
+        if (c < d) {
+          const float4 a = *reinterpret_cast<const float4*>(b.delta + base + c + p * b.plane);
+          v[i].x += a.x; v[i].y += a.y; v[i].z += a.z; v[i].w += a.w;
+        }
+      }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < VMAX; ++i) ss += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+    const float f = rsqrtf(block_sum4(ss, red) / (float)d + eps);
+#pragma unroll
+    for (int i = 0; i < VMAX; ++i) {
+      acc[i].x += v[i].x * f * wv[i].x * inv;
+      acc[i].y += v[i].y * f * wv[i].y * inv;
+      acc[i].z += v[i].z * f * wv[i].z * inv;
+      acc[i].w += v[i].w * f * wv[i].w * inv;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < VMAX; ++i) {
+    const int c = 4 * (threadIdx.x + 256 * i);
+    if (c < d) *reinterpret_cast<float4*>(out + base + c) = acc[i];
+  }
+}
+
 // deltas[i]: [planes[i], nt, d] float32, ``plane[i]`` elements apart; ws[i]: [d]; out [nt, d].
 extern "C" int ta_normed_mean(hipStream_t stream, int n, const float* const* deltas, const int* planes,
                               const long long* plane, const float* const* ws, float eps, float* out, int nt, int d) {
@@ -239,6 +328,12 @@ extern "C" int ta_normed_mean(hipStream_t stream, int n, const float* const* del
     br.b[i] = MeanBranch{deltas[i], ws[i], plane[i], planes[i]};
   }
   if (nt == 0) return 0;
-  normed_mean_kernel<<<nt, 256, 0, stream>>>(br, n, eps, out, d);
+  bool vec = d % 4 == 0 && d <= 4096 && (uintptr_t)out % 16 == 0;
+  for (int i = 0; i < n; ++i)
+    vec = vec && plane[i] % 4 == 0 && (uintptr_t)deltas[i] % 16 == 0 && (uintptr_t)ws[i] % 16 == 0;
+  if (vec)
+    normed_mean_vec_kernel<<<nt, 256, 0, stream>>>(br, n, eps, out, d);
+  else
+    normed_mean_kernel<<<nt, 256, 0, stream>>>(br, n, eps, out, d);
   return ta_check_launch("ta_normed_mean");
 }
