@@ -825,45 +825,56 @@ __global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o
   }
 }
 
-// The same for wide heads (all heads normed as one row of thousands of columns): four waves share
-// a row, each thread keeps its columns in registers.
+// The same for wide heads (all heads normed as one row of thousands of columns): eight waves share
+// a row, each thread keeps its columns in registers. Four planes are asked for at once, and the
+// gate and the weight before the sum over the row is known, so that a row of a single-token step
+// waits for memory twice, not once per plane.
 template <typename T>
-__global__ __launch_bounds__(256) void gla_out_wide_kernel(const float* __restrict__ o, int parts, size_t plane,
+__global__ __launch_bounds__(512) void gla_out_wide_kernel(const float* __restrict__ o, int parts, size_t plane,
                                                            const T* __restrict__ proj, int stride,
                                                            const float* __restrict__ w, int wstride, float eps,
                                                            int H, int dv, T* __restrict__ out, int gate_act) {
-  constexpr int PER = 16;                 // columns a thread can own: rows of up to 256 * PER
-  __shared__ float red[4];
+  constexpr int PER = 8;                  // columns a thread can own: rows of up to 512 * PER
+  __shared__ float red[8];
   const size_t t = blockIdx.x;
   const int h = blockIdx.y;
   const float* src = o + (t * H + h) * dv;
-  float v[PER];
-  float ss = 0.f;
+  float v[PER], g[PER], wc[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) v[i] = 0.f;
+  for (int p0 = 0; p0 < parts; p0 += 4) {
+    float a[4][PER];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int c = threadIdx.x + 512 * i;
+        a[q][i] = (c < dv && p0 + q < parts) ? src[(size_t)(p0 + q) * plane + c] : 0.f;
+      }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)           // planes in order: the sum does not depend on how they are fetched
+#pragma unroll
+      for (int i = 0; i < PER; ++i) v[i] += a[q][i];
+  }
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
-    const int c = threadIdx.x + 256 * i;
-    v[i] = c < dv ? src[c] : 0.f;
+    const int c = threadIdx.x + 512 * i;
+    g[i] = c < dv ? to_f32(proj[t * stride + h * dv + c]) : 0.f;
+    wc[i] = (c < dv && w) ? w[h * wstride + c] : 1.0f;
   }
-  for (int p = 1; p < parts; ++p)
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      if (c < dv) v[i] += src[p * plane + c];
-    }
+  float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < PER; ++i) ss += v[i] * v[i];
   ss = wave_sum(ss);
   if (threadIdx.x % TA_WAVE == 0) red[threadIdx.x / TA_WAVE] = ss;
   __syncthreads();
-  const float f = rsqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)dv + eps);
+  const float f = rsqrtf((((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]))) / (float)dv + eps);
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
-    const int c = threadIdx.x + 256 * i;
+    const int c = threadIdx.x + 512 * i;
     if (c < dv) {
-      const float g = to_f32(proj[t * stride + h * dv + c]);
-      const float sg = 1.0f / (1.0f + expf(-g));
-      const float wc = w ? w[h * wstride + c] : 1.0f;
-      out[t * (size_t)(H * dv) + h * dv + c] = from_f32<T>(v[i] * f * wc * (gate_act == 1 ? sg : g * sg));
+      const float sg = 1.0f / (1.0f + expf(-g[i]));
+      out[t * (size_t)(H * dv) + h * dv + c] = from_f32<T>(v[i] * f * wc[i] * (gate_act == 1 ? sg : g[i] * sg));
     }
   }
 }
@@ -883,9 +894,9 @@ extern "C" int ta_gla_out_act(hipStream_t stream, int dtype, const float* o, int
   const size_t plane = (size_t)nt * H * dv, lds = (size_t)dv * sizeof(float);
   if (dv > 512 && dv <= 4096 && (dtype == TA_F32 || dtype == TA_BF16)) {
     if (dtype == TA_F32)
-      gla_out_wide_kernel<float><<<g, 256, 0, stream>>>(o, parts, plane, (const float*)proj + goff, stride, w, wstride, eps, H, dv, (float*)out, gate_act);
+      gla_out_wide_kernel<float><<<g, 512, 0, stream>>>(o, parts, plane, (const float*)proj + goff, stride, w, wstride, eps, H, dv, (float*)out, gate_act);
     else
-      gla_out_wide_kernel<bf16_t><<<g, 256, 0, stream>>>(o, parts, plane, (const bf16_t*)proj + goff, stride, w, wstride, eps, H, dv, (bf16_t*)out, gate_act);
+      gla_out_wide_kernel<bf16_t><<<g, 512, 0, stream>>>(o, parts, plane, (const bf16_t*)proj + goff, stride, w, wstride, eps, H, dv, (bf16_t*)out, gate_act);
     return ta_check_launch("ta_gla_out");
   }
   if (dtype == TA_F32)
