@@ -123,7 +123,7 @@ def test_router_bias_and_softmax_over_the_chosen(geom):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("geom", [(5, 2, 24, 72, 40, 1.0, 0.7), (3, 3, 16, 72, None, 2.0, 0.0), (1, 1, 32, 64, 8, 1.0, 1.0),
-                                  (7, 1, 20, 90, 12, 0.5, 3.0), (16, 2, 64, 320, 128, 1.5, 1.0), (8, 2, 256, 1024, 512, 1.5, 1.0)])
+                                  (7, 1, 20, 90, 12, 0.5, 3.0), (12, 3, 48, 328, 96, 1.25, 0.9), (8, 2, 256, 1024, 512, 1.5, 1.0)])
 def test_routed_limited_experts_part(dtype, geom):
     """The routed feed-forward as the block runs it (routing with the bias, ordering, both products,
     the limited gate, the shared expert, the other sublayer's delta taken into the sum) against the
