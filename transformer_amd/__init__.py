@@ -1,4 +1,4 @@
-"""A small decoder engine for one MI355X (Llama, Vametar, Kunitar, Luduvik): typed configuration, weights by name,
+"""A small decoder engine for one MI355X (Llama, Vametar, Kunitar, Luduvik, Saredra): typed configuration, weights by name,
 blocks assembled from parts, a paged per-sequence cache, one batched step
 function, a generation loop, sampling and trace replay, on hand-written HIP
 kernels for gfx950."""
@@ -9,6 +9,7 @@ from .config.llama import LlamaConfig  # noqa: F401
 from .config.vametar import VametarConfig  # noqa: F401
 from .config.kunitar import KunitarConfig  # noqa: F401
 from .config.luduvik import LuduvikConfig  # noqa: F401
+from .config.saredra import SaredraConfig  # noqa: F401
 from .config.registry import get_architecture, known_architectures, register_architecture  # noqa: F401
 from .parts.base import PartTimers, register_part  # noqa: F401
 from .llama import Llama  # noqa: F401

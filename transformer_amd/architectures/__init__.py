@@ -1,2 +1,2 @@
 """Registry entries. Importing the package registers them."""
-from . import kunitar, llama, luduvik, vametar  # noqa: F401
+from . import kunitar, llama, luduvik, saredra, vametar  # noqa: F401

@@ -42,6 +42,13 @@ class PositionSpec:
     # are divided by factor, those below original/high stay, and between the two the share of
     # the unscaled frequency grows linearly in original/wavelength from 0 to 1
     scaling: Optional[Tuple[float, float, float, float]] = None
+    # (factor, original, fast, slow) or None: another way to slow the long wavelengths, a ramp over
+    # the pair index i. n(t) = head_dim * ln(original / (2 pi t)) / (2 ln theta) is the index at
+    # which t turns fit into ``original`` positions; lo = max(floor(n(fast)), 0), hi = min(ceil(n(slow)),
+    # head_dim - 1), r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), and f_i <- f_i / factor * r_i +
+    # f_i * (1 - r_i). ``scaling`` and ``ramp`` exclude each other.
+    ramp: Optional[Tuple[float, float, float, float]] = None
+    magnitude: float = 1.0      # cos and sin are both multiplied by it
 
 
 @dataclass(frozen=True)
@@ -72,11 +79,12 @@ class SwiGLUSpec:
 
 @dataclass(frozen=True)
 class BlockSpec:
-    """x += mixer(norm1(x)); x += ffn(norm2(x))  (kind "prenorm")."""
+    """x += mixer(norm1(x)); x += ffn(norm2(x))  (kind "prenorm"). ffn None (and norm2 None): the
+    block has the mixer only."""
     norm1: object
     mixer: object
-    norm2: object
-    ffn: object
+    norm2: object = None
+    ffn: object = None
     kind: str = "prenorm"
 
 
@@ -316,12 +324,18 @@ class RoutedMLPSpec:
     # form "mlp": down(act(up(h))). form "limited_glu": an expert has a gate and an up matrix,
     # g = min(gate(h), limit), u = clamp(up(h), -limit, limit), down(g * sigmoid(gate_slope * g)
     # * (u + up_shift)); ``activation`` is not used then. shared_limit: the shared expert's limit.
+    # form "glu": an expert is down(act(gate(h)) * up(h)) with ``activation`` "silu" or "gelu_tanh", its
+    # first matrix [gate rows | up rows] as in "limited_glu".
+    # groups > 1: the experts form that many equal groups of neighbours; a group counts as the
+    # largest score in it, and only experts of the ``keep_groups`` best groups can be chosen.
     router_bias: bool = False
     form: str = "mlp"
     limit: float = 0.0
     shared_limit: float = 0.0
     gate_slope: float = 1.702
     up_shift: float = 1.0
+    groups: int = 1
+    keep_groups: int = 1
 
 
 @dataclass(frozen=True)
@@ -439,3 +453,78 @@ class ParallelBlockSpec:
     mixer: object
     ffn: object = None
     kind: str = "parallel_prenorm"
+
+
+# ---------------------------------------------------------------------------------------------
+# Parts that the Saredra decoder added; as above, every size and constant is a field.
+
+@dataclass(frozen=True)
+class SinkAttentionSpec:
+    """Causal grouped-query softmax attention with key and value widths of their own, whose scores
+    may be capped and whose softmax denominator may hold one more term.
+
+    score = q . k * scale; softcap: score <- softcap * tanh(score / softcap). window: a query at p
+    reads keys in (p - window, p]; None: all. sink None: plain softmax; "unit": the denominator also
+    holds exp(0) = 1; "learned": exp(s_h) with a learned s_h per head; the extra term has no value.
+    rot_dims: the first coordinates of every head of q and k that turn by position * f_i, f_i =
+    rot_base^(-2i/rot_dims), in pairs of ``rot_style`` ("interleaved": (2i, 2i + 1); "half": (i, i +
+    rot_dims/2)); rot_ramp / rot_magnitude: see ``PositionSpec.ramp`` / ``.magnitude``.
+    qkv_bias: q, k, v have biases, added in the projection. conv_taps > 0: a causal convolution of that
+    many taps per channel (no bias, no activation) on q, k and v between projection and rotation; the
+    last taps - 1 projected rows of a sequence are carried between steps. out_gate: the concatenated
+    heads are multiplied by sigmoid(Wg h) before the output projection. own_kv False: no key and value
+    projections; the layer reads what the layer whose cache it borrows stored (its schedule entry
+    names it). cache_window: the window the cache layer is kept for (the widest of the layers that
+    read it; None: everything)."""
+    hidden: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    softcap: Optional[float] = None
+    window: Optional[int] = None
+    cache_window: Optional[int] = None
+    sink: Optional[str] = None
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_style: str = "interleaved"
+    rot_ramp: Optional[Tuple[float, float, float, float]] = None
+    rot_magnitude: float = 1.0
+    qkv_bias: bool = False
+    conv_taps: int = 0
+    out_gate: bool = False
+    own_kv: bool = True
+    kind: str = "attention_sink"
+
+
+@dataclass(frozen=True)
+class StateSpaceSpec:
+    """A selective state-space mixer with a scalar decay per head (state-space duality).
+
+    inner = num_heads * head_dim. One projection gives [z: inner | x: inner | B: groups * state | C:
+    groups * state | dt: num_heads]; x, B and C pass a causal convolution of ``taps`` per channel (with
+    bias) and silu; dt <- softplus(dt + dt_bias). Per head h of group h // (num_heads / groups): S_t =
+    exp(-exp(A_log_h) dt_t) S_(t-1) + dt_t B_t x_t^T (S is [state, head_dim], float32, zero at a
+    sequence's start), y_t = S_t^T C_t + D_h x_t. y * silu(z) is RMS-normed in ``norm_groups`` equal
+    parts of the row (each by its own root mean square), times a weight, then projected."""
+    hidden: int
+    num_heads: int
+    head_dim: int
+    state: int
+    groups: int
+    taps: int
+    norm_groups: int
+    eps: float
+    kind: str = "state_space"
+
+
+@dataclass(frozen=True)
+class BranchSumSpec:
+    """Several mixers side by side that read the same rows: the result is sum_i scales[i] *
+    branches[i](h). names[i] prefixes the parameters of branches[i]."""
+    hidden: int
+    branches: Tuple[object, ...]
+    names: Tuple[str, ...]
+    scales: Tuple[float, ...]
+    kind: str = "branch_sum"

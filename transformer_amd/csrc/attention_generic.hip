@@ -29,7 +29,8 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
     const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
-    const int* __restrict__ pos0, int nh, int nkv, int dh, int dv, float scale, int window) {
+    const int* __restrict__ pos0, int nh, int nkv, int dh, int dv, float scale, int window,
+    float softcap, int sink_mode, const float* __restrict__ sink, const T* __restrict__ gate, int gate_stride) {
   extern __shared__ float smem[];
   const int group = nh / nkv;
   const int b = blockIdx.z, kvh = blockIdx.y;
@@ -104,8 +105,14 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     const int kk0 = key0 + lane, kk1 = kk0 + 16;
     const bool v0 = row_ok && kk0 >= my_start && kk0 < my_end;
     const bool v1 = row_ok && kk1 >= my_start && kk1 < my_end;
-    s0 = v0 ? s0 * scale : -INFINITY;
-    s1 = v1 ? s1 * scale : -INFINITY;
+    s0 *= scale;
+    s1 *= scale;
+    if (softcap > 0.f) {              // capped scores: cap * tanh(score / cap)
+      s0 = softcap * tanhf(s0 / softcap);
+      s1 = softcap * tanhf(s1 / softcap);
+    }
+    s0 = v0 ? s0 : -INFINITY;
+    s1 = v1 ? s1 : -INFINITY;
     const float m_new = fmaxf(m, group16_max(fmaxf(s0, s1)));
     float alpha = 1.f, e0 = 0.f, e1 = 0.f;
     if (m_new != -INFINITY) {
@@ -139,11 +146,26 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     __syncthreads();
   }
   if (row_ok) {
+    // a sink is one more term of the denominator with a score of its own and no value:
+    // sink_mode 1: score 0 for every head; 2: sink[head]
+    if (sink_mode != 0) {
+      const float sv = sink_mode == 2 ? sink[head] : 0.f;
+      const float m_new = fmaxf(m, sv);
+      const float alpha = expf(m - m_new);          // m = -inf (no key seen) gives 0
+      l = l * alpha + expf(sv - m_new);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] *= alpha;
+    }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     T* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * dv + lane;
+    const T* gt = gate ? gate + (size_t)(q0 + qi) * gate_stride + (size_t)head * dv + lane : nullptr;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
-      if (i < nd && 16 * i + lane < dv) o[16 * i] = from_f32<T>(acc[i] * inv);
+      if (i < nd && 16 * i + lane < dv) {
+        float r = acc[i] * inv;
+        if (gt) r *= 1.0f / (1.0f + expf(-to_f32(gt[16 * i])));      // the heads' sigmoid gate
+        o[16 * i] = from_f32<T>(r);
+      }
   }
 }
 
@@ -157,8 +179,13 @@ static int attention_generic_launch(hipStream_t stream, int dtype, const void* q
                                     void* out, int out_stride, const void* kcache,
                                     const void* vcache, const int* block_table, int max_blocks,
                                     const int* cu_q, const int* pos0, int batch, int max_qlen,
-                                    int nh, int nkv, int dh, int dv, float scale, int window) {
+                                    int nh, int nkv, int dh, int dv, float scale, int window,
+                                    float softcap = 0.f, int sink_mode = 0, const float* sink = nullptr,
+                                    const void* gate = nullptr, int gate_stride = 0) {
   TA_REQUIRE(batch >= 0 && max_qlen >= 0, "ta_attention_generic: bad batch=%d max_qlen=%d", batch, max_qlen);
+  TA_REQUIRE(sink_mode >= 0 && sink_mode <= 2 && (sink_mode != 2 || sink != nullptr) && softcap >= 0.f,
+             "ta_attention_generic: sink mode %d, cap %f", sink_mode, softcap);
+  TA_REQUIRE(gate == nullptr || gate_stride >= nh * dv, "ta_attention_generic: gate rows of %d", gate_stride);
   TA_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "ta_attention_generic: %d heads do not divide into %d kv heads", nh, nkv);
   TA_REQUIRE(dh >= 1 && dh <= 256 && dv >= 1 && dv <= 256,
              "ta_attention_generic: key width %d / value width %d outside [1, 256]", dh, dv);
@@ -172,11 +199,13 @@ static int attention_generic_launch(hipStream_t stream, int dtype, const void* q
   if (dtype == TA_F32)
     attn_generic_kernel<float><<<g, blk, lds, stream>>>(
         (const float*)q, q_stride, (float*)out, out_stride, (const float*)kcache,
-        (const float*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, dv, scale, window);
+        (const float*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, dv, scale, window,
+        softcap, sink_mode, sink, (const float*)gate, gate_stride);
   else if (dtype == TA_BF16)
     attn_generic_kernel<bf16_t><<<g, blk, lds, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
-        (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, dv, scale, window);
+        (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, dv, scale, window,
+        softcap, sink_mode, sink, (const bf16_t*)gate, gate_stride);
   else
     return ta_fail("ta_attention_generic: unknown dtype %d", dtype);
   return ta_check_launch("ta_attention_generic");
@@ -199,4 +228,19 @@ extern "C" int ta_attention_generic_dv(hipStream_t stream, int dtype, const void
                                        int nh, int nkv, int dh, int dv, float scale, int window) {
   return attention_generic_launch(stream, dtype, q, q_stride, out, out_stride, kcache, vcache, block_table,
                                   max_blocks, cu_q, pos0, batch, max_qlen, nh, nkv, dh, dv, scale, window);
+}
+
+// The same with the options of a capped, sunk and gated softmax: softcap > 0: score <- softcap *
+// tanh(score / softcap) after the scale; sink_mode 1: the denominator holds one more term exp(0);
+// 2: exp(sink[head]) (float32 [nh]); gate: rows [nt, >= nh*dv] whose sigmoid multiplies the result.
+extern "C" int ta_attention_generic_sink(hipStream_t stream, int dtype, const void* q, int q_stride,
+                                         void* out, int out_stride, const void* kcache,
+                                         const void* vcache, const int* block_table, int max_blocks,
+                                         const int* cu_q, const int* pos0, int batch, int max_qlen,
+                                         int nh, int nkv, int dh, int dv, float scale, int window,
+                                         float softcap, int sink_mode, const float* sink, const void* gate,
+                                         int gate_stride) {
+  return attention_generic_launch(stream, dtype, q, q_stride, out, out_stride, kcache, vcache, block_table,
+                                  max_blocks, cu_q, pos0, batch, max_qlen, nh, nkv, dh, dv, scale, window,
+                                  softcap, sink_mode, sink, gate, gate_stride);
 }

@@ -316,3 +316,80 @@ extern "C" int ta_qk_prepare(hipStream_t stream, int dtype, void* qkv, int strid
     return ta_fail("ta_qk_prepare: unknown dtype %d", dtype);
   return ta_check_launch("ta_qk_prepare");
 }
+
+// ------------------------------------------------------------------ rotation and cache write, no norm
+// Rows [q | k | v] (nh*dk, nkv*dk, nkv*dv columns; a layer that reads another layer's keys and values
+// has q only: nkv_own = 0). bias [columns] float32 or null is added first. The first `rot` coordinates
+// of every head of q and k turn by the token's angles cs [nt, rot/2] (cos, sin): style 0 pairs
+// (i, i + rot/2), style 1 pairs (2i, 2i + 1). q goes back in place; k and v go to the paged cache at
+// dest[t] (keys [pages][kv heads][PAGE][dk], values [pages][kv heads][dv][PAGE]). float32 inside, one
+// rounding of each result. One workgroup per token, a thread per pair of coordinates.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_rotate_store_kernel(
+    T* __restrict__ qkv, int stride, const float* __restrict__ bias, const float2* __restrict__ cs, int rot,
+    int style, const int* __restrict__ dest, T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv,
+    int nkv_own, int dk, int dv) {
+  const int t = blockIdx.x;
+  T* row = qkv + (size_t)t * stride;
+  const int nq = nh * dk, nk = nkv_own * dk, nv = nkv_own * dv;
+  const int half = rot / 2, hd2 = dk / 2;              // dk is even
+  const float2* ang = cs ? cs + (size_t)t * half : nullptr;
+  const int page = dest ? dest[t] / TA_PAGE : 0, off = dest ? dest[t] % TA_PAGE : 0;
+  for (int i = threadIdx.x; i < (nq + nk) / 2; i += 256) {
+    const int head = i / hd2, p = i - head * hd2;      // pair p of head (q heads first, then k heads)
+    int c0, c1;
+    bool turns = ang != nullptr && p < half;
+    if (style == 1) { c0 = 2 * p; c1 = 2 * p + 1; }
+    else if (p < half) { c0 = p; c1 = p + half; }
+    else {                                              // the coordinates that no pair of style 0 covers
+      const int r = p - half;                           // rot + 2r, rot + 2r + 1
+      c0 = rot + 2 * r; c1 = c0 + 1;
+    }
+    const int base = head * dk;
+    float u = to_f32(row[base + c0]), v = to_f32(row[base + c1]);
+    if (bias) { u += bias[base + c0]; v += bias[base + c1]; }
+    if (turns) {
+      const float2 a = ang[p];
+      const float nu = u * a.x - v * a.y, nv2 = v * a.x + u * a.y;
+      u = nu; v = nv2;
+    }
+    if (head < nh) {
+      row[base + c0] = from_f32<T>(u);
+      row[base + c1] = from_f32<T>(v);
+    } else if (dest) {
+      T* kd = kcache + (((size_t)page * nkv + (head - nh)) * TA_PAGE + off) * dk;
+      kd[c0] = from_f32<T>(u);
+      kd[c1] = from_f32<T>(v);
+    }
+  }
+  if (dest) {
+    for (int i = threadIdx.x; i < nv; i += 256) {
+      float v = to_f32(row[nq + nk + i]);
+      if (bias) v += bias[nq + nk + i];
+      const int g = i / dv, c = i - g * dv;
+      vcache[(((size_t)page * nkv + g) * dv + c) * TA_PAGE + off] = from_f32<T>(v);
+    }
+  }
+}
+
+extern "C" int ta_qk_rotate_store(hipStream_t stream, int dtype, void* qkv, int stride, const float* bias,
+                                  const float* cs, int rot, int style, const int* dest, void* kcache, void* vcache,
+                                  int nt, int nh, int nkv, int nkv_own, int dk, int dv) {
+  TA_REQUIRE(nt >= 0 && nh >= 1 && nkv >= 1 && (nkv_own == 0 || nkv_own == nkv) && dk >= 2 && dk % 2 == 0 && dv >= 1,
+             "ta_qk_rotate_store: bad sizes nt=%d heads=%d/%d (%d own) widths %d/%d", nt, nh, nkv, nkv_own, dk, dv);
+  TA_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dk && (rot == 0 || cs != nullptr) && (style == 0 || style == 1),
+             "ta_qk_rotate_store: %d rotated coordinates of %d, style %d", rot, dk, style);
+  TA_REQUIRE(stride >= nh * dk + nkv_own * (dk + dv), "ta_qk_rotate_store: rows of %d are too short", stride);
+  TA_REQUIRE(dest == nullptr || (nkv_own == nkv && kcache && vcache), "ta_qk_rotate_store: a cache write needs keys, values and a cache");
+  if (nt == 0) return 0;
+  if (dtype == TA_F32)
+    qk_rotate_store_kernel<float><<<nt, 256, 0, stream>>>((float*)qkv, stride, bias, rot ? (const float2*)cs : nullptr,
+                                                          rot, style, dest, (float*)kcache, (float*)vcache, nh, nkv,
+                                                          nkv_own, dk, dv);
+  else if (dtype == TA_BF16)
+    qk_rotate_store_kernel<bf16_t><<<nt, 256, 0, stream>>>((bf16_t*)qkv, stride, bias, rot ? (const float2*)cs : nullptr,
+                                                           rot, style, dest, (bf16_t*)kcache, (bf16_t*)vcache, nh, nkv,
+                                                           nkv_own, dk, dv);
+  else return ta_fail("ta_qk_rotate_store: unknown dtype %d", dtype);
+  return ta_check_launch("ta_qk_rotate_store");
+}

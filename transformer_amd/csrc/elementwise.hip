@@ -289,22 +289,28 @@ extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype
 // Angles of a step: cs[t][j] = (cos a, sin a), a = (float)pos[t] * inv_freq[j] formed
 // in float32. Every layer with the same frequencies shares the table of the step.
 __global__ void rope_table_kernel(const int* __restrict__ pos, const float* __restrict__ inv_freq,
-                                  float2* __restrict__ cs, int half) {
+                                  float2* __restrict__ cs, int half, float magnitude) {
   const int t = blockIdx.x;
   const float p = (float)pos[t];
   for (int j = threadIdx.x; j < half; j += blockDim.x) {
     float sn, c;
     sincosf(p * inv_freq[j], &sn, &c);
-    cs[(size_t)t * half + j] = make_float2(c, sn);
+    cs[(size_t)t * half + j] = make_float2(c * magnitude, sn * magnitude);
   }
+}
+
+// magnitude: both cos and sin are multiplied by it (1 for a plain rotation).
+extern "C" int ta_rope_table_scaled(hipStream_t stream, const int* pos, const float* inv_freq, float* cs,
+                                    int nt, int half, float magnitude) {
+  TA_REQUIRE(nt >= 0 && half > 0, "ta_rope_table: bad sizes nt=%d half=%d", nt, half);
+  if (nt == 0) return 0;
+  rope_table_kernel<<<nt, 64, 0, stream>>>(pos, inv_freq, (float2*)cs, half, magnitude);
+  return ta_check_launch("ta_rope_table");
 }
 
 extern "C" int ta_rope_table(hipStream_t stream, const int* pos, const float* inv_freq, float* cs,
                              int nt, int half) {
-  TA_REQUIRE(nt >= 0 && half > 0, "ta_rope_table: bad sizes nt=%d half=%d", nt, half);
-  if (nt == 0) return 0;
-  rope_table_kernel<<<nt, 64, 0, stream>>>(pos, inv_freq, (float2*)cs, half);
-  return ta_check_launch("ta_rope_table");
+  return ta_rope_table_scaled(stream, pos, inv_freq, cs, nt, half, 1.0f);
 }
 
 // qkv: [nt, nq + 2*nkv, dh]. Per token t:

@@ -24,12 +24,14 @@
 // logits: [nt, ld] float32, the first E columns of a row are the router's. mode 0: sigmoid
 // scores; 1: softmax over the experts. renorm: the chosen weights are divided by their sum
 // (with mode 1 that is the softmax over the chosen logits alone). bias [E] or null: added to
-// the logits first.
+// the logits first. groups > 1: the experts form that many equal groups of neighbours, a group
+// counts as its largest score, and only experts of the `keep` best groups (the lowest index
+// among equals) can be chosen.
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int ld, int E, int top,
                                                        int mode, int renorm, int* __restrict__ chosen,
                                                        float* __restrict__ weight,
-                                                       const float* __restrict__ bias) {
-  extern __shared__ float sc[];           // [E]
+                                                       const float* __restrict__ bias, int groups, int keep) {
+  extern __shared__ float sc[];           // [E], then a score per group [groups]
   const size_t t = blockIdx.x;
   const int lane = threadIdx.x;
   float mx = -INFINITY;
@@ -44,6 +46,25 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
   }
   sum = wave_sum(sum);
   __syncthreads();
+  if (groups > 1) {
+    float* gs = sc + E;
+    const int size = E / groups;
+    for (int g = lane; g < groups; g += 64) {
+      float best = -INFINITY;
+      for (int e = g * size; e < (g + 1) * size; ++e) best = fmaxf(best, sc[e]);
+      gs[g] = best;
+    }
+    __syncthreads();
+    // a group stays when fewer than `keep` groups come before it in the order (score down, index up)
+    for (int g = lane; g < groups; g += 64) {
+      const float mine = gs[g];
+      int ahead = 0;
+      for (int o = 0; o < groups; ++o) ahead += (gs[o] > mine || (gs[o] == mine && o < g)) ? 1 : 0;
+      if (ahead >= keep)
+        for (int e = g * size; e < (g + 1) * size; ++e) sc[e] = -INFINITY;
+    }
+    __syncthreads();
+  }
   float total = 0.f;
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
@@ -74,13 +95,21 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
   }
 }
 
-extern "C" int ta_moe_route_bias(hipStream_t stream, const float* logits, const float* bias, int ld, int nt, int E,
-                                 int top, int mode, int renorm, int* chosen, float* weight) {
+extern "C" int ta_moe_route_groups(hipStream_t stream, const float* logits, const float* bias, int ld, int nt, int E,
+                                   int top, int mode, int renorm, int groups, int keep, int* chosen, float* weight) {
   TA_REQUIRE(nt >= 0 && E >= 1 && E <= 8192 && top >= 1 && top <= E && ld >= E && (mode == 0 || mode == 1),
              "ta_moe_route: bad sizes nt=%d experts=%d top=%d ld=%d", nt, E, top, ld);
+  TA_REQUIRE(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (E / groups),
+             "ta_moe_route: %d experts in %d groups of which %d stay do not hold %d choices", E, groups, keep, top);
   if (nt == 0) return 0;
-  moe_route_kernel<<<nt, 64, (size_t)E * sizeof(float), stream>>>(logits, ld, E, top, mode, renorm, chosen, weight, bias);
+  moe_route_kernel<<<nt, 64, (size_t)(E + groups) * sizeof(float), stream>>>(logits, ld, E, top, mode, renorm, chosen,
+                                                                             weight, bias, groups, keep);
   return ta_check_launch("ta_moe_route");
+}
+
+extern "C" int ta_moe_route_bias(hipStream_t stream, const float* logits, const float* bias, int ld, int nt, int E,
+                                 int top, int mode, int renorm, int* chosen, float* weight) {
+  return ta_moe_route_groups(stream, logits, bias, ld, nt, E, top, mode, renorm, 1, 1, chosen, weight);
 }
 
 extern "C" int ta_moe_route(hipStream_t stream, const float* logits, int ld, int nt, int E, int top, int mode,

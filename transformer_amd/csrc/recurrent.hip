@@ -569,7 +569,9 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
     const T* __restrict__ proj, int stride, int qoff, int koff, int voff, const float* __restrict__ alpha,
     float qscale, float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots,
     int H, int dk, int dv, int col_tiles, size_t plane, float* __restrict__ o_out,
-    const float* __restrict__ bonus, const float* __restrict__ head_decay) {
+    const float* __restrict__ bonus, const float* __restrict__ head_decay,
+    int qk_share = 1, const float* __restrict__ tok_decay = nullptr,
+    const float* __restrict__ tok_kscale = nullptr) {
   __shared__ float sq[GLA_TC][GLA_RT], sk[GLA_TC][GLA_RT], sa[GLA_TC][GLA_RT];
   __shared__ float sv[GLA_TC][GLA_CT];
   __shared__ float part[GLA_TC][4][GLA_CT];
@@ -600,6 +602,9 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
   }
   // one fixed decay for all key channels of the head (``alpha`` is then not read)
   const float fixed = head_decay ? head_decay[h] : 0.f;
+  // qk_share consecutive heads read the same q and k (one group of them); tok_decay / tok_kscale
+  // [nt, H]: one decay for all key channels of (token, head), and a factor on that token's key
+  const int hq = h / qk_share;
   // Loads are asked for two chunks ahead (a trip to memory takes longer than a chunk's
   // arithmetic); a position that is not there reads a harmless address and is replaced.
   auto fetch = [&](GlaOperands<GLA_TC>& o, int t0) {
@@ -609,11 +614,13 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
       const bool ok = t0 + tt < end && i < dk;
       const size_t row = (size_t)(ok ? t0 + tt : start);
       const int ii = ok ? i : 0;
-      const float qv = to_f32(proj[row * stride + qoff + h * dk + ii]);
-      const float kv = to_f32(proj[row * stride + koff + h * dk + ii]);
-      const float av = head_decay ? fixed : alpha[row * ((size_t)H * dk) + h * dk + ii];
+      const float qv = to_f32(proj[row * stride + qoff + hq * dk + ii]);
+      const float kv = to_f32(proj[row * stride + koff + hq * dk + ii]);
+      const float av = head_decay ? fixed : tok_decay ? tok_decay[row * H + h]
+                                                      : alpha[row * ((size_t)H * dk) + h * dk + ii];
+      const float ks = tok_kscale ? tok_kscale[row * H + h] : 1.f;
       o.q[e] = ok ? qv * qscale : 0.f;
-      o.k[e] = ok ? kv : 0.f;
+      o.k[e] = ok ? kv * ks : 0.f;
       o.a[e] = ok ? av : 1.f;           // a token that is not there leaves S as it is
     }
 #pragma unroll
@@ -721,10 +728,12 @@ static int gla_recurrent_launch(hipStream_t stream, int dtype, int wdtype, const
                                 const void* a2, const float* a2b, float inv_tau, float qscale, float* alpha,
                                 float* state, const int* cu_q, const int* slots, int batch, int nt, int H, int dk,
                                 int dv, float* o_out, int mode, const float* bonus,
-                                const float* head_decay = nullptr) {
+                                const float* head_decay = nullptr, int qk_share = 1,
+                                const float* tok_decay = nullptr, const float* tok_kscale = nullptr) {
   TA_REQUIRE(batch > 0 && batch <= 65535 && H > 0 && H <= 65535 && nt >= batch,
              "ta_gla_recurrent: bad batch %d / heads %d / tokens %d", batch, H, nt);
-  TA_REQUIRE(dk >= 1 && dv >= 1 && (head_decay || (rank >= 1 && rank <= 8192)),
+  TA_REQUIRE(qk_share >= 1 && H % qk_share == 0, "ta_gla_recurrent: %d heads do not form groups of %d", H, qk_share);
+  TA_REQUIRE(dk >= 1 && dv >= 1 && (head_decay || tok_decay || (rank >= 1 && rank <= 8192)),
              "ta_gla_recurrent: bad widths %d / %d / %d", dk, dv, rank);
   const int parts = (dk + GLA_RT - 1) / GLA_RT, tiles = (dv + GLA_CT - 1) / GLA_CT;
   TA_REQUIRE(parts * tiles <= 65535, "ta_gla_recurrent: heads of %d x %d are too large", dk, dv);
@@ -733,7 +742,7 @@ static int gla_recurrent_launch(hipStream_t stream, int dtype, int wdtype, const
   const size_t lds = (size_t)rank * sizeof(float);
 #define GLA_DECAY(T, TW) \
   gla_decay_kernel<T, TW><<<gd, 256, lds, stream>>>((const T*)low, low_stride, aoff, rank, (const TW*)a2, a2b, inv_tau, n, alpha, mode)
-  if (head_decay) {
+  if (head_decay || tok_decay) {
     TA_REQUIRE(dtype == TA_F32 || dtype == TA_BF16, "ta_gla_recurrent: unknown dtype %d", dtype);
   } else if (dtype == TA_F32 && wdtype == TA_F32) GLA_DECAY(float, float);
   else if (dtype == TA_BF16 && wdtype == TA_BF16) GLA_DECAY(bf16_t, bf16_t);
@@ -746,7 +755,7 @@ static int gla_recurrent_launch(hipStream_t stream, int dtype, int wdtype, const
 #define GLA_RUN(T, TC, B)                                                                                   \
   gla_recurrent_kernel<T, TC, B><<<g, 256, 0, stream>>>((const T*)proj, stride, qoff, koff, voff, alpha, qscale, \
                                                         state, cu_q, slots, H, dk, dv, tiles, plane, o_out, bonus, \
-                                                        head_decay)
+                                                        head_decay, qk_share, tok_decay, tok_kscale)
   if (bonus) {
     if (dtype == TA_F32) {
       if (few) GLA_RUN(float, 8, true); else GLA_RUN(float, 32, true);
@@ -918,4 +927,191 @@ extern "C" int ta_gla_out_w(hipStream_t stream, int dtype, const float* o, int p
 extern "C" int ta_gla_out(hipStream_t stream, int dtype, const float* o, int parts, const void* proj, int stride,
                           int goff, const float* w, float eps, int nt, int H, int dv, void* out) {
   return ta_gla_out_w(stream, dtype, o, parts, proj, stride, goff, w, 0, eps, nt, H, dv, out);
+}
+
+// ------------------------------------------------------------------ short causal convolution
+// y_t[c] = act(bias_out[c] + sum_j taps[c][j] * u_{t-(K-1-j)}[c]) on a range of columns of the rows
+// of ``in``; u = in + bias_in (a bias that belongs to the projection in front). Inputs before a
+// sequence's first token of the step come from conv_state [slots, K-1, C] float32 (zero for a new
+// sequence), which `conv_state_update` replaces afterwards by the step's last K-1 inputs.
+// Sums are float32; act 0: none, 1: silu.
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_kernel(
+    const T* __restrict__ in, int stride, int off, const float* __restrict__ bias_in,
+    const float* __restrict__ taps, const float* __restrict__ bias_out, const float* __restrict__ conv_state,
+    const int* __restrict__ tok_seq, const int* __restrict__ cu_q, const int* __restrict__ slots, int C, int K,
+    int act, T* __restrict__ out, int out_stride) {
+  const int t = blockIdx.x;
+  const int b = tok_seq[t];
+  const int start = cu_q[b];
+  const size_t slot = (size_t)slots[b];
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
+    const float bi = bias_in ? bias_in[c] : 0.f;
+    float acc = bias_out ? bias_out[c] : 0.f;
+    for (int j = 0; j < K; ++j) {
+      const int src = t - (K - 1 - j);
+      float u;
+      if (src >= start) u = to_f32(in[(size_t)src * stride + off + c]) + bi;
+      else u = conv_state[(slot * (K - 1) + (K - 1 - (start - src))) * C + c];
+      acc = fmaf(taps[(size_t)c * K + j], u, acc);
+    }
+    if (act == 1) acc = acc / (1.0f + expf(-acc));
+    out[(size_t)t * out_stride + c] = from_f32<T>(acc);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(
+    const T* __restrict__ in, int stride, int off, const float* __restrict__ bias_in, float* __restrict__ conv_state,
+    const int* __restrict__ cu_q, const int* __restrict__ slots, int C, int K) {
+  const int b = blockIdx.x;
+  const int start = cu_q[b], n = cu_q[b + 1] - start;
+  const size_t slot = (size_t)slots[b];
+  float* st = conv_state + slot * (K - 1) * C;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
+    const float bi = bias_in ? bias_in[c] : 0.f;
+    // new row r holds the input n - (K-1) + r of the step, or the old row r + n where that is negative;
+    // rows are rewritten in ascending order and every read is of a row at or behind the one written
+    for (int r = 0; r < K - 1; ++r) {
+      const int src = n - (K - 1) + r;
+      const float v = src >= 0 ? to_f32(in[(size_t)(start + src) * stride + off + c]) + bi : st[(size_t)(r + n) * C + c];
+      st[(size_t)r * C + c] = v;
+    }
+  }
+}
+
+__global__ void token_sequence_kernel(const int* __restrict__ cu_q, int batch, int* __restrict__ tok_seq) {
+  const int b = blockIdx.x;
+  for (int t = cu_q[b] + threadIdx.x; t < cu_q[b + 1]; t += blockDim.x) tok_seq[t] = b;
+}
+
+// tok_seq [nt] int32 scratch: the sequence of every token of the step (filled here from cu_q).
+// in: [nt, stride] rows, the convolution reads columns off .. off + C; out: [nt, out_stride] rows,
+// columns 0 .. C. taps [C, K] float32; bias_in, bias_out [C] float32 or null; conv_state [slots, K-1, C]
+// float32 (null with K == 1: no memory). update 0: the state is left as it is.
+extern "C" int ta_causal_conv(hipStream_t stream, int dtype, const void* in, int stride, int off,
+                              const float* bias_in, const float* taps, const float* bias_out, float* conv_state,
+                              int* tok_seq, const int* cu_q, const int* slots, int batch, int nt, int C, int K,
+                              int act, void* out, int out_stride, int update) {
+  TA_REQUIRE(batch > 0 && batch <= 65535 * 32 && nt >= batch && C >= 1 && K >= 1 && K <= 64,
+             "ta_causal_conv: bad sizes batch=%d nt=%d channels=%d taps=%d", batch, nt, C, K);
+  TA_REQUIRE(off >= 0 && stride >= off + C && out_stride >= C && (act == 0 || act == 1),
+             "ta_causal_conv: columns %d..%d of rows of %d, out rows of %d, act %d", off, off + C, stride, out_stride, act);
+  TA_REQUIRE(K == 1 || conv_state != nullptr, "ta_causal_conv: %d taps need the sequences' memory", K);
+  token_sequence_kernel<<<batch, 256, 0, stream>>>(cu_q, batch, tok_seq);
+  const int cb = (C + 255) / 256 < 64 ? (C + 255) / 256 : 64;
+  dim3 g(nt, cb), gs(batch, cb);
+#define CONV_RUN(T)                                                                                              \
+  do {                                                                                                           \
+    causal_conv_kernel<T><<<g, 256, 0, stream>>>((const T*)in, stride, off, bias_in, taps, bias_out, conv_state, \
+                                                 tok_seq, cu_q, slots, C, K, act, (T*)out, out_stride);         \
+    if (update && K > 1)                                                                                         \
+      conv_state_update_kernel<T><<<gs, 256, 0, stream>>>((const T*)in, stride, off, bias_in, conv_state, cu_q,  \
+                                                          slots, C, K);                                          \
+  } while (0)
+  if (dtype == TA_F32) CONV_RUN(float);
+  else if (dtype == TA_BF16) CONV_RUN(bf16_t);
+  else return ta_fail("ta_causal_conv: unknown dtype %d", dtype);
+#undef CONV_RUN
+  return ta_check_launch("ta_causal_conv");
+}
+
+// ------------------------------------------------------------------ selective state space
+// Step sizes and decays of every (token, head), float32: dt = softplus(raw + dt_bias[h]) (no clamp),
+// decay = exp(-exp(a_log[h]) * dt).
+template <typename T>
+__global__ __launch_bounds__(256) void ssm_steps_kernel(const T* __restrict__ proj, int stride, int off,
+                                                        const float* __restrict__ dt_bias,
+                                                        const float* __restrict__ a_log, int nt, int H,
+                                                        float* __restrict__ dt, float* __restrict__ decay) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)nt * H) return;
+  const size_t t = i / H;
+  const int h = (int)(i - t * H);
+  const float z = to_f32(proj[t * stride + off + h]) + dt_bias[h];
+  const float sp = fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));
+  dt[i] = sp;
+  decay[i] = expf(-expf(a_log[h]) * sp);
+}
+
+extern "C" int ta_ssm_steps(hipStream_t stream, int dtype, const void* proj, int stride, int off,
+                            const float* dt_bias, const float* a_log, int nt, int H, float* dt, float* decay) {
+  TA_REQUIRE(nt >= 0 && H >= 1 && off >= 0 && stride >= off + H, "ta_ssm_steps: bad sizes nt=%d heads=%d", nt, H);
+  if (nt == 0) return 0;
+  const unsigned blocks = (unsigned)(((size_t)nt * H + 255) / 256);
+  if (dtype == TA_F32)
+    ssm_steps_kernel<float><<<blocks, 256, 0, stream>>>((const float*)proj, stride, off, dt_bias, a_log, nt, H, dt, decay);
+  else if (dtype == TA_BF16)
+    ssm_steps_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)proj, stride, off, dt_bias, a_log, nt, H, dt, decay);
+  else return ta_fail("ta_ssm_steps: unknown dtype %d", dtype);
+  return ta_check_launch("ta_ssm_steps");
+}
+
+// The recurrence S_t = decay_t S_{t-1} + dt_t B_t x_t^T, o_t = S_t^T C_t per head, with B and C shared
+// by the ``share`` heads of a group: the kernel of gated linear attention with q = C, k = B, v = x,
+// one decay per (token, head) and the step size as a factor on the key. decay, dt: [nt, H] float32.
+extern "C" int ta_ssm_recurrent(hipStream_t stream, int dtype, const void* proj, int stride, int coff, int boff,
+                                int xoff, int share, const float* decay, const float* dt, float* state,
+                                const int* cu_q, const int* slots, int batch, int nt, int H, int N, int P,
+                                float* o_out) {
+  TA_REQUIRE(decay != nullptr && dt != nullptr, "ta_ssm_recurrent: decays and step sizes are required");
+  return gla_recurrent_launch(stream, dtype, dtype, proj, stride, coff, boff, xoff, nullptr, 0, 0, 0, nullptr,
+                              nullptr, 1.0f, 1.0f, nullptr, state, cu_q, slots, batch, nt, H, N, P, o_out, 0,
+                              nullptr, nullptr, share, decay, dt);
+}
+
+// y = (sum of the readout's planes + skip[h] * x) * silu(z), cut into ``groups`` equal parts of the row,
+// each divided by its own root mean square, times w: the gate comes BEFORE the norm. One wave a
+// (token, part); float32 inside. o: [parts, nt, n]; x at column xoff of xs rows, z at zoff of zs rows.
+template <typename T>
+__global__ __launch_bounds__(64) void gated_group_norm_kernel(
+    const float* __restrict__ o, int parts, size_t plane, const T* __restrict__ xs, int x_stride, int xoff,
+    const float* __restrict__ skip, int head_dim, const T* __restrict__ zs, int z_stride, int zoff,
+    const float* __restrict__ w, float eps, int n, int groups, T* __restrict__ out) {
+  const size_t t = blockIdx.x;
+  const int g = blockIdx.y, len = n / groups, c0 = g * len;
+  const int lane = threadIdx.x;
+  float ss = 0.f;
+  for (int c = c0 + lane; c < c0 + len; c += 64) {
+    float y = 0.f;
+    for (int p = 0; p < parts; ++p) y += o[p * plane + t * n + c];
+    if (skip) y = fmaf(skip[c / head_dim], to_f32(xs[t * x_stride + xoff + c]), y);
+    const float z = to_f32(zs[t * z_stride + zoff + c]);
+    y *= z / (1.0f + expf(-z));
+    ss = fmaf(y, y, ss);
+  }
+  ss = wave_sum(ss);
+  const float f = rsqrtf(ss / (float)len + eps);
+  for (int c = c0 + lane; c < c0 + len; c += 64) {
+    float y = 0.f;
+    for (int p = 0; p < parts; ++p) y += o[p * plane + t * n + c];
+    if (skip) y = fmaf(skip[c / head_dim], to_f32(xs[t * x_stride + xoff + c]), y);
+    const float z = to_f32(zs[t * z_stride + zoff + c]);
+    y *= z / (1.0f + expf(-z));
+    out[t * n + c] = from_f32<T>(y * f * (w ? w[c] : 1.f));
+  }
+}
+
+extern "C" int ta_gated_group_norm(hipStream_t stream, int dtype, const float* o, int parts, const void* xs,
+                                   int x_stride, int xoff, const float* skip, int head_dim, const void* zs,
+                                   int z_stride, int zoff, const float* w, float eps, int nt, int n, int groups,
+                                   void* out) {
+  TA_REQUIRE(nt >= 0 && n >= 1 && groups >= 1 && groups <= 65535 && n % groups == 0 && parts >= 1,
+             "ta_gated_group_norm: rows of %d in %d parts, %d planes", n, groups, parts);
+  TA_REQUIRE(skip == nullptr || (head_dim >= 1 && n % head_dim == 0 && x_stride >= xoff + n),
+             "ta_gated_group_norm: heads of %d in rows of %d", head_dim, n);
+  TA_REQUIRE(z_stride >= zoff + n, "ta_gated_group_norm: gate rows of %d", z_stride);
+  if (nt == 0) return 0;
+  dim3 g(nt, groups);
+  const size_t plane = (size_t)nt * n;
+  if (dtype == TA_F32)
+    gated_group_norm_kernel<float><<<g, 64, 0, stream>>>(o, parts, plane, (const float*)xs, x_stride, xoff, skip,
+                                                         head_dim, (const float*)zs, z_stride, zoff, w, eps, n, groups,
+                                                         (float*)out);
+  else if (dtype == TA_BF16)
+    gated_group_norm_kernel<bf16_t><<<g, 64, 0, stream>>>(o, parts, plane, (const bf16_t*)xs, x_stride, xoff, skip,
+                                                          head_dim, (const bf16_t*)zs, z_stride, zoff, w, eps, n, groups,
+                                                          (bf16_t*)out);
+  else return ta_fail("ta_gated_group_norm: unknown dtype %d", dtype);
+  return ta_check_launch("ta_gated_group_norm");
 }

@@ -337,3 +337,42 @@ extern "C" int ta_normed_mean(hipStream_t stream, int n, const float* const* del
     normed_mean_kernel<<<nt, 256, 0, stream>>>(br, n, eps, out, d);
   return ta_check_launch("ta_normed_mean");
 }
+
+// ------------------------------------------------------------------ weighted sum of branches
+// out = sum over i of scale[i] * (sum of the planes of deltas[i]); float32, 1 to 4 branches.
+struct SumBranches {
+  const float* d[4];
+  long long plane[4];
+  int planes[4];
+  float scale[4];
+};
+
+__global__ __launch_bounds__(256) void weighted_sum_kernel(SumBranches br, int n, float* __restrict__ out, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+    float acc = 0.f;
+    for (int b = 0; b < n; ++b) {
+      float s = 0.f;
+      for (int p = 0; p < br.planes[b]; ++p) s += br.d[b][(size_t)p * br.plane[b] + i];
+      acc = fmaf(br.scale[b], s, acc);
+    }
+    out[i] = acc;
+  }
+}
+
+// deltas[i]: [planes[i], nt, d] float32, ``plane[i]`` elements apart; out [nt, d].
+extern "C" int ta_weighted_sum(hipStream_t stream, int n, const float* const* deltas, const int* planes,
+                               const long long* plane, const float* scales, float* out, int nt, int d) {
+  TA_REQUIRE(n >= 1 && n <= 4, "ta_weighted_sum: %d branches (1 to 4 are taken)", n);
+  TA_REQUIRE(nt >= 0 && d > 0, "ta_weighted_sum: bad sizes nt=%d d=%d", nt, d);
+  SumBranches br;
+  for (int i = 0; i < 4; ++i) { br.d[i] = nullptr; br.plane[i] = 0; br.planes[i] = 0; br.scale[i] = 0.f; }
+  for (int i = 0; i < n; ++i) {
+    TA_REQUIRE(deltas[i] && planes[i] >= 1 && planes[i] <= TA_MAX_PLANES, "ta_weighted_sum: branch %d: %d planes", i, planes[i]);
+    br.d[i] = deltas[i]; br.plane[i] = plane[i]; br.planes[i] = planes[i]; br.scale[i] = scales[i];
+  }
+  if (nt == 0) return 0;
+  const size_t total = (size_t)nt * d;
+  const unsigned blocks = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+  weighted_sum_kernel<<<blocks, 256, 0, stream>>>(br, n, out, total);
+  return ta_check_launch("ta_weighted_sum");
+}

@@ -150,15 +150,16 @@ def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Te
 
 
 # ------------------------------------------------------------------ rotary + cache write
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t, j] = (cos a, sin a) with a = float32(positions[t]) * inv_freq[j] in float32."""
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor,
+               magnitude: float = 1.0) -> torch.Tensor:
+    """out[t, j] = magnitude * (cos a, sin a) with a = float32(positions[t]) * inv_freq[j] in float32."""
     _dev(positions, "positions", torch.int32); _dev(inv_freq, "inv_freq", torch.float32)
     _dev(out, "out", torch.float32)
     nt, half = positions.numel(), inv_freq.numel()
     if tuple(out.shape) != (nt, half, 2):
         raise KernelError(f"rope_table: out is {tuple(out.shape)}, expected {(nt, half, 2)}")
-    _check(library().ta_rope_table(_stream(), _ptr(positions), _ptr(inv_freq), _ptr(out), c_int(nt),
-                                   c_int(half)))
+    _check(library().ta_rope_table_scaled(_stream(), _ptr(positions), _ptr(inv_freq), _ptr(out), c_int(nt),
+                                          c_int(half), c_float(magnitude)))
     return out
 
 
@@ -1563,11 +1564,14 @@ def moe_max_rows(pairs: int, experts: int) -> int:
 
 
 def moe_route(logits: torch.Tensor, experts: int, top: int, chosen: torch.Tensor, weight: torch.Tensor,
-              score: str = "sigmoid", renormalize: bool = False, bias: Optional[torch.Tensor] = None):
+              score: str = "sigmoid", renormalize: bool = False, bias: Optional[torch.Tensor] = None,
+              groups: int = 1, keep_groups: int = 1):
     """chosen [nt, top] int32, weight [nt, top] float32: the ``top`` largest scores of the
     first ``experts`` columns of logits [nt, >= experts] float32 (lowest index among equals).
     bias [experts] float32: added to the logits first. "softmax" with ``renormalize`` is the
-    softmax over the chosen logits alone."""
+    softmax over the chosen logits alone. groups > 1: the experts form that many equal groups of
+    neighbours, a group counts as its largest score, and only experts of the ``keep_groups`` best
+    groups can be chosen."""
     _dev(logits, "logits", torch.float32, contiguous=False)
     nt, ld = _rows2d(logits, "logits")
     _dev(chosen, "chosen", torch.int32); _dev(weight, "weight", torch.float32)
@@ -1577,9 +1581,12 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, chosen: torch.Tensor
         _dev(bias, "bias", torch.float32)
         if bias.shape != (experts,):
             raise KernelError(f"moe_route: bias is {tuple(bias.shape)}, expected {(experts,)}")
-    _check(library().ta_moe_route_bias(_stream(), _ptr(logits), _ptr(bias), c_int(ld), c_int(nt), c_int(experts),
-                                       c_int(top), c_int(_ROUTE_MODES[score]), c_int(int(renormalize)),
-                                       _ptr(chosen), _ptr(weight)))
+    if groups < 1 or experts % groups or not 1 <= keep_groups <= groups or top > keep_groups * (experts // groups):
+        raise KernelError(f"moe_route: {experts} experts in {groups} groups of which {keep_groups} stay "
+                          f"do not hold {top} choices")
+    _check(library().ta_moe_route_groups(_stream(), _ptr(logits), _ptr(bias), c_int(ld), c_int(nt), c_int(experts),
+                                         c_int(top), c_int(_ROUTE_MODES[score]), c_int(int(renormalize)),
+                                         c_int(groups), c_int(keep_groups), _ptr(chosen), _ptr(weight)))
     return chosen, weight
 
 
@@ -1667,3 +1674,246 @@ def moe_combine(rows: torch.Tensor, top: int, pair_row: torch.Tensor, weight, sh
                                           c_int(gl), _ptr(extra), c_int(xplanes), c_longlong(xplane), _ptr(delta),
                                           c_int(nt)))
     return delta
+
+
+# ------------------------------------------------------------------ capped, sunk and gated softmax attention
+_ROT_STYLES = {"half": 0, "interleaved": 1}
+
+
+def qk_rotate_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int,
+                    own_kv: bool = True, bias: Optional[torch.Tensor] = None, angles: Optional[torch.Tensor] = None,
+                    rot: int = 0, style: str = "interleaved", dest: Optional[torch.Tensor] = None,
+                    kcache: Optional[torch.Tensor] = None, vcache: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """On rows [q | k | v] of ``qkv`` (nh*dk, nkv*dk, nkv*dv columns; q alone without ``own_kv``):
+    ``bias`` [columns] float32 is added, the first ``rot`` coordinates of every head of q and k turn by
+    ``angles`` [nt, rot/2, 2] ("half": pairs (i, i + rot/2); "interleaved": (2i, 2i + 1)), q goes back
+    in place, k and v are stored at ``dest`` into the cache layer (values of their own width)."""
+    _dev(qkv, "qkv", contiguous=False)
+    nt, stride = _rows2d(qkv, "qkv")
+    own = num_kv_heads if own_kv else 0
+    cols = num_heads * key_dim + own * (key_dim + value_dim)
+    if qkv.shape[1] != cols:
+        raise KernelError(f"qk_rotate_store: rows of {qkv.shape[1]}, expected {cols}")
+    if style not in _ROT_STYLES or key_dim % 2 or rot % 2 or not 0 <= rot <= key_dim:
+        raise KernelError(f"qk_rotate_store: {rot} rotated coordinates of heads of {key_dim}, pairing {style!r}")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.shape != (cols,):
+            raise KernelError(f"qk_rotate_store: bias is {tuple(bias.shape)}, expected {(cols,)}")
+    if rot:
+        _dev(angles, "angles", torch.float32)
+        if tuple(angles.shape) != (nt, rot // 2, 2):
+            raise KernelError(f"qk_rotate_store: angles are {tuple(angles.shape)}, expected {(nt, rot // 2, 2)}")
+    else:
+        angles = None
+    if dest is not None:
+        if not own_kv:
+            raise KernelError("qk_rotate_store: a layer without keys and values of its own stores nothing")
+        _dev(dest, "dest", torch.int32); _dev(kcache, "kcache", qkv.dtype); _dev(vcache, "vcache", qkv.dtype)
+        _check_cache_layer("qk_rotate_store", kcache, vcache, num_kv_heads, key_dim, value_dim)
+        if dest.numel() != nt:
+            raise KernelError("qk_rotate_store: dest must hold one entry per token")
+    _check(library().ta_qk_rotate_store(
+        _stream(), c_int(_code(qkv.dtype)), _ptr(qkv), c_int(stride), _ptr(bias), _ptr(angles), c_int(rot),
+        c_int(_ROT_STYLES[style]), _ptr(dest), _ptr(kcache if dest is not None else None),
+        _ptr(vcache if dest is not None else None), c_int(nt), c_int(num_heads), c_int(num_kv_heads), c_int(own),
+        c_int(key_dim), c_int(value_dim)))
+    return qkv
+
+
+def attention_sink(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads, num_kv_heads, key_dim,
+                   value_dim, scale, window=None, softcap: Optional[float] = None, sink=None,
+                   gate: Optional[torch.Tensor] = None):
+    """``attention_generic_dv`` with the options of a capped, sunk and gated softmax. softcap: score <-
+    softcap * tanh(score / softcap) after the scale. sink: None; "unit": the denominator holds one more
+    term exp(0) = 1; a float32 tensor [heads]: one more term exp(sink[head]). gate: rows [nt, >= heads *
+    value_dim] of q's type whose sigmoid multiplies the result element by element."""
+    _dev(q, "q", contiguous=False); _dev(out, "out", q.dtype, contiguous=False)
+    nt, qs = _rows2d(q, "q")
+    nto, os_ = _rows2d(out, "out")
+    if nt != nto or q.shape[1] < num_heads * key_dim or out.shape[1] != num_heads * value_dim:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit "
+                          f"{num_heads} heads of {key_dim} / {value_dim}")
+    _dev(kcache, "kcache", q.dtype); _dev(vcache, "vcache", q.dtype)
+    _check_cache_layer("attention", kcache, vcache, num_kv_heads, key_dim, value_dim)
+    _dev(block_table, "block_table", torch.int32); _dev(cu_q, "cu_q", torch.int32)
+    _dev(pos0, "pos0", torch.int32)
+    B = pos0.numel()
+    if cu_q.numel() != B + 1 or block_table.dim() != 2 or block_table.shape[0] != B:
+        raise KernelError("attention: cu_q / pos0 / block_table disagree about the batch size")
+    mode, sink_t = 0, None
+    if isinstance(sink, str):
+        if sink != "unit":
+            raise KernelError(f"attention: unknown sink {sink!r}")
+        mode = 1
+    elif sink is not None:
+        _dev(sink, "sink", torch.float32)
+        if sink.shape != (num_heads,):
+            raise KernelError(f"attention: sink is {tuple(sink.shape)}, expected {(num_heads,)}")
+        mode, sink_t = 2, sink
+    gs = 0
+    if gate is not None:
+        _dev(gate, "gate", q.dtype, contiguous=False)
+        ng, gs = _rows2d(gate, "gate")
+        if ng != nt or gate.shape[1] < num_heads * value_dim:
+            raise KernelError(f"attention: gate rows are {tuple(gate.shape)}")
+    if softcap is not None and not softcap > 0:
+        raise KernelError(f"attention: a cap must be positive, got {softcap}")
+    _check(library().ta_attention_generic_sink(
+        _stream(), c_int(_code(q.dtype)), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache),
+        _ptr(vcache), _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0),
+        c_int(B), c_int(max_qlen), c_int(num_heads), c_int(num_kv_heads), c_int(key_dim),
+        c_int(value_dim), c_float(scale), c_int(window or 0), c_float(softcap or 0.0), c_int(mode),
+        _ptr(sink_t), _ptr(gate), c_int(gs)))
+    return out
+
+
+# ------------------------------------------------------------------ short convolution, selective state space
+_CONV_ACTS = {None: 0, "silu": 1}
+
+
+def causal_conv(x: torch.Tensor, offset: int, channels: int, taps: torch.Tensor, out: torch.Tensor,
+                conv_state: Optional[torch.Tensor], cu_q: torch.Tensor, slots: torch.Tensor, tok_seq: torch.Tensor,
+                bias_in: Optional[torch.Tensor] = None, bias_out: Optional[torch.Tensor] = None,
+                activation: Optional[str] = None, update: bool = True) -> torch.Tensor:
+    """out[t, c] = act(bias_out[c] + sum_j taps[c, j] * u_(t - K + 1 + j)[c]) per sequence, u = columns
+    [offset, offset + channels) of the rows of ``x`` plus ``bias_in``. Inputs before the step's first
+    token of a sequence come from conv_state [slots, K - 1, channels] float32 (zero for a new sequence),
+    which afterwards holds the sequence's last K - 1 inputs (``update``). taps [channels, K] float32;
+    out [nt, channels] of x's type, not x itself; tok_seq: int32 scratch [nt]."""
+    _dev(x, "x", contiguous=False); _dev(out, "out", x.dtype, contiguous=False)
+    nt, stride = _rows2d(x, "x")
+    nto, ostride = _rows2d(out, "out")
+    _dev(taps, "taps", torch.float32)
+    if taps.dim() != 2 or taps.shape[0] != channels or nto != nt or out.shape[1] != channels or \
+            offset < 0 or offset + channels > x.shape[1]:
+        raise KernelError(f"causal_conv: x {tuple(x.shape)} columns {offset}..{offset + channels}, taps "
+                          f"{tuple(taps.shape)}, out {tuple(out.shape)}")
+    K = taps.shape[1]
+    if activation not in _CONV_ACTS:
+        raise KernelError(f"causal_conv: unknown activation {activation!r}")
+    for name, b in (("bias_in", bias_in), ("bias_out", bias_out)):
+        if b is not None:
+            _dev(b, name, torch.float32)
+            if b.shape != (channels,):
+                raise KernelError(f"causal_conv: {name} is {tuple(b.shape)}, expected {(channels,)}")
+    batch = _step_tables(cu_q, slots, nt, "causal_conv")
+    if K > 1:
+        _dev(conv_state, "conv_state", torch.float32)
+        if conv_state.dim() != 3 or tuple(conv_state.shape[1:]) != (K - 1, channels):
+            raise KernelError(f"causal_conv: state is {tuple(conv_state.shape)}, expected [slots, {K - 1}, {channels}]")
+    _dev(tok_seq, "tok_seq", torch.int32)
+    if tok_seq.numel() < nt:
+        raise KernelError("causal_conv: tok_seq holds one entry per token")
+    if out.data_ptr() == x.data_ptr():
+        raise KernelError("causal_conv: the result needs rows of its own")
+    _check(library().ta_causal_conv(
+        _stream(), c_int(_code(x.dtype)), _ptr(x), c_int(stride), c_int(offset), _ptr(bias_in), _ptr(taps),
+        _ptr(bias_out), _ptr(conv_state if K > 1 else None), _ptr(tok_seq), _ptr(cu_q), _ptr(slots), c_int(batch),
+        c_int(nt), c_int(channels), c_int(K), c_int(_CONV_ACTS[activation]), _ptr(out), c_int(ostride),
+        c_int(int(update))))
+    return out
+
+
+def ssm_steps(proj: torch.Tensor, offset: int, heads: int, dt_bias: torch.Tensor, a_log: torch.Tensor,
+              dt: torch.Tensor, decay: torch.Tensor):
+    """dt[t, h] = softplus(proj[t, offset + h] + dt_bias[h]) (no clamp), decay[t, h] = exp(-exp(a_log[h]) *
+    dt[t, h]); both float32 [nt, heads]."""
+    _dev(proj, "proj", contiguous=False)
+    nt, stride = _rows2d(proj, "proj")
+    _dev(dt_bias, "dt_bias", torch.float32); _dev(a_log, "a_log", torch.float32)
+    _dev(dt, "dt", torch.float32); _dev(decay, "decay", torch.float32)
+    if dt_bias.shape != (heads,) or a_log.shape != (heads,) or dt.shape != (nt, heads) or decay.shape != (nt, heads) \
+            or offset < 0 or offset + heads > proj.shape[1]:
+        raise KernelError(f"ssm_steps: proj {tuple(proj.shape)} columns {offset}..{offset + heads}, "
+                          f"dt {tuple(dt.shape)}, decay {tuple(decay.shape)}")
+    _check(library().ta_ssm_steps(_stream(), c_int(_code(proj.dtype)), _ptr(proj), c_int(stride), c_int(offset),
+                                  _ptr(dt_bias), _ptr(a_log), c_int(nt), c_int(heads), _ptr(dt), _ptr(decay)))
+    return dt, decay
+
+
+def ssm_recurrent(xbc: torch.Tensor, x_off: int, b_off: int, c_off: int, heads: int, groups: int, state_dim: int,
+                  head_dim: int, decay: torch.Tensor, dt: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
+                  slots: torch.Tensor, o_out: torch.Tensor) -> torch.Tensor:
+    """Per head h of group h // (heads / groups): S_t = decay[t, h] S_(t-1) + dt[t, h] B_t x_t^T (S is
+    [state_dim, head_dim], float32, in ``state`` [slots, heads, state_dim, head_dim]), o_t = S_t^T C_t.
+    x (heads * head_dim columns), B and C (groups * state_dim each) sit at column offsets of the rows of
+    ``xbc``. o_out: [gla_row_parts(state_dim), nt, heads, head_dim] float32 planes that add up to o."""
+    _dev(xbc, "xbc", contiguous=False)
+    nt, stride = _rows2d(xbc, "xbc")
+    if groups < 1 or heads % groups:
+        raise KernelError(f"ssm_recurrent: {heads} heads do not divide into {groups} groups")
+    for off, n in ((x_off, heads * head_dim), (b_off, groups * state_dim), (c_off, groups * state_dim)):
+        if off < 0 or off + n > xbc.shape[1]:
+            raise KernelError(f"ssm_recurrent: columns {off}..{off + n} of rows of {xbc.shape[1]}")
+    _dev(decay, "decay", torch.float32); _dev(dt, "dt", torch.float32)
+    _dev(state, "state", torch.float32); _dev(o_out, "o_out", torch.float32)
+    if decay.shape != (nt, heads) or dt.shape != (nt, heads):
+        raise KernelError(f"ssm_recurrent: decay {tuple(decay.shape)} / dt {tuple(dt.shape)}, expected {(nt, heads)}")
+    if state.dim() != 4 or tuple(state.shape[1:]) != (heads, state_dim, head_dim):
+        raise KernelError(f"ssm_recurrent: state is {tuple(state.shape)}")
+    if tuple(o_out.shape) != (gla_row_parts(state_dim), nt, heads, head_dim):
+        raise KernelError(f"ssm_recurrent: o_out is {tuple(o_out.shape)}")
+    batch = _step_tables(cu_q, slots, nt, "ssm_recurrent")
+    _check(library().ta_ssm_recurrent(
+        _stream(), c_int(_code(xbc.dtype)), _ptr(xbc), c_int(stride), c_int(c_off), c_int(b_off), c_int(x_off),
+        c_int(heads // groups), _ptr(decay), _ptr(dt), _ptr(state), _ptr(cu_q), _ptr(slots), c_int(batch), c_int(nt),
+        c_int(heads), c_int(state_dim), c_int(head_dim), _ptr(o_out)))
+    return o_out
+
+
+def gated_group_norm(o: torch.Tensor, gate: torch.Tensor, gate_off: int, weight: Optional[torch.Tensor], eps: float,
+                     groups: int, out: torch.Tensor, x: Optional[torch.Tensor] = None, x_off: int = 0,
+                     skip: Optional[torch.Tensor] = None, head_dim: int = 0) -> torch.Tensor:
+    """y = (sum of the planes of o + skip[head] * x) * silu(gate); the row is cut into ``groups`` equal
+    parts, each divided by its own root mean square, times weight: the gate comes before the norm.
+    o float32 [planes, nt, n]; gate at column gate_off of its rows, x at x_off of its rows (same type
+    as out); skip float32 [n / head_dim]; out [nt, n]."""
+    _dev(o, "o", torch.float32); _dev(out, "out")
+    if o.dim() != 3 or out.dim() != 2 or tuple(o.shape[1:]) != tuple(out.shape):
+        raise KernelError(f"gated_group_norm: o {tuple(o.shape)} / out {tuple(out.shape)}")
+    parts, nt, n = o.shape
+    if groups < 1 or n % groups:
+        raise KernelError(f"gated_group_norm: rows of {n} do not divide into {groups} parts")
+    _dev(gate, "gate", out.dtype, contiguous=False)
+    ng, gs = _rows2d(gate, "gate")
+    if ng != nt or gate_off < 0 or gate_off + n > gate.shape[1]:
+        raise KernelError(f"gated_group_norm: gate rows {tuple(gate.shape)}, columns {gate_off}..{gate_off + n}")
+    xs = 0
+    if skip is not None:
+        _dev(skip, "skip", torch.float32); _dev(x, "x", out.dtype, contiguous=False)
+        nx, xs = _rows2d(x, "x")
+        if head_dim < 1 or n % head_dim or skip.shape != (n // head_dim,) or nx != nt or x_off < 0 or x_off + n > x.shape[1]:
+            raise KernelError(f"gated_group_norm: skip {tuple(skip.shape)} for heads of {head_dim} in rows of {n}")
+    if weight is not None:
+        _dev(weight, "weight", torch.float32)
+        if weight.shape != (n,):
+            raise KernelError(f"gated_group_norm: weight is {tuple(weight.shape)}, expected {(n,)}")
+    _check(library().ta_gated_group_norm(
+        _stream(), c_int(_code(out.dtype)), _ptr(o), c_int(parts), _ptr(x if skip is not None else None), c_int(xs),
+        c_int(x_off), _ptr(skip), c_int(head_dim), _ptr(gate), c_int(gs), c_int(gate_off), _ptr(weight), c_float(eps),
+        c_int(nt), c_int(n), c_int(groups), _ptr(out)))
+    return out
+
+
+def weighted_sum(deltas: Sequence[torch.Tensor], scales: Sequence[float], out: torch.Tensor) -> torch.Tensor:
+    """out = sum over i of scales[i] * deltas[i]: deltas float32 [nt, d] or [planes, nt, d] (planes added
+    in order), out float32 [nt, d]."""
+    _dev(out, "out", torch.float32)
+    nt, d = out.shape
+    n = len(deltas)
+    if not 1 <= n <= 4 or len(scales) != n:
+        raise KernelError(f"weighted_sum: {n} branches with {len(scales)} scales (1 to 4 are taken)")
+    planes, plane = [], []
+    for i, t in enumerate(deltas):
+        _dev(t, f"deltas[{i}]", torch.float32)
+        if t.dim() == 3 and t.shape[1:] == out.shape:
+            planes.append(t.shape[0]); plane.append(nt * d)
+        elif t.shape == out.shape:
+            planes.append(1); plane.append(0)
+        else:
+            raise KernelError(f"weighted_sum: deltas[{i}] is {tuple(t.shape)}, out {tuple(out.shape)}")
+    dp = (c_void_p * n)(*[t.data_ptr() for t in deltas])
+    _check(library().ta_weighted_sum(_stream(), c_int(n), dp, (c_int * n)(*planes), (c_longlong * n)(*plane),
+                                     (c_float * n)(*[float(v) for v in scales]), _ptr(out), c_int(nt), c_int(d)))
+    return out

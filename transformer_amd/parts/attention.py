@@ -244,3 +244,97 @@ class NormedAttention(Part):
 
 
 register_part("attention_normed", NormedAttention)
+
+
+class SinkAttention(Part):
+    """Softmax attention with key and value widths of their own, capped scores, a window and one
+    more term in the softmax denominator (``SinkAttentionSpec``).
+
+    One merged product gives [q | k | v | gate] (k and v only where the layer has keys and values of
+    its own, the gate only where the heads are gated). Where the spec names a convolution, q, k and
+    v pass it channel by channel (``kernels.causal_conv``, which keeps a sequence's last projected
+    rows between steps). ``kernels.qk_rotate_store`` adds the biases where there is no convolution to
+    take them, turns q and k and writes k and v to the paged cache; ``kernels.attention_sink`` reads
+    the cache with scores, cap, sink, softmax and sums in float32 and applies the heads' gate; the
+    output projection follows. A layer that borrows reads the lender's cache layer through its
+    schedule entry and declares the same need."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        s = spec
+        if s.num_heads % s.num_kv_heads:
+            raise PartError(f"{s.num_heads} heads do not divide into {s.num_kv_heads} kv heads")
+        if not (2 <= s.key_dim <= 256 and s.key_dim % 2 == 0 and 1 <= s.value_dim <= 256):
+            raise PartError(f"attention takes even key widths and value widths in [1, 256], not {s.key_dim} / {s.value_dim}")
+        if s.rot_dims % 2 or not 0 <= s.rot_dims <= s.key_dim or s.rot_style not in ("half", "interleaved"):
+            raise PartError(f"{s.rot_dims} rotated coordinates ({s.rot_style!r}) do not fit heads of {s.key_dim}")
+        if s.window is not None and s.window < 1:
+            raise PartError(f"attention window must be >= 1, got {s.window}")
+        if s.cache_window is not None and (s.window is None or s.cache_window < s.window):
+            raise PartError(f"a cache kept for {s.cache_window} tokens does not serve a window of {s.window}")
+        if s.sink not in (None, "unit", "learned"):
+            raise PartError(f"unknown sink {s.sink!r}")
+        if s.softcap is not None and not s.softcap > 0:
+            raise PartError(f"a score cap must be positive, got {s.softcap}")
+        if s.conv_taps < 0 or (s.conv_taps and not s.own_kv):
+            raise PartError("a convolution on q, k and v needs keys and values of the layer's own")
+        self.spec, self.dtype = s, dtype
+        self.nq, self.nkv, self.dk, self.dv = s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim
+        self.qkv_width = self.nq * self.dk + (self.nkv * (self.dk + self.dv) if s.own_kv else 0)
+        self.width = self.qkv_width + (self.nq * self.dv if s.out_gate else 0)
+        self.rotary = None
+        if s.rot_dims:
+            from ..config.spec import PositionSpec
+            self.rotary = build_part(PositionSpec(head_dim=s.rot_dims, theta=s.rot_base, style=s.rot_style,
+                                                  ramp=s.rot_ramp, magnitude=s.rot_magnitude), dtype, device)
+
+    def params(self):
+        s = self.spec
+        p = {"in.weight": Param((self.width, s.hidden), "matrix"),        # q, k, v, gate
+             "out.weight": Param((s.hidden, self.nq * self.dv), "matrix")}
+        if s.qkv_bias:
+            p["in.bias"] = Param((self.qkv_width,), "vector")
+        if s.conv_taps:
+            p["conv.weight"] = Param((self.qkv_width, s.conv_taps), "vector")
+        if s.sink == "learned":
+            p["sink"] = Param((self.nq,), "vector", init="zero")
+        return p
+
+    def cache_need(self):
+        s = self.spec
+        window = s.window if s.cache_window is None else s.cache_window
+        kv = KVNeed(self.nkv, self.dk, window, self.dv)
+        if s.conv_taps > 1:
+            from ..cache.storage import StateNeed
+            return [kv, StateNeed((s.conv_taps - 1, self.qkv_width), torch.float32)]
+        return kv
+
+    def run(self, h, ctx, cache, layer, writes_cache=True):
+        s, nt = self.spec, h.shape[0]
+        if not s.own_kv and writes_cache:
+            raise PartError("a layer without keys and values of its own runs on another layer's cache")
+        proj = linear(h, self.w["in.weight"], ctx.ws.take("attention.in", (nt, self.width), self.dtype))
+        kv_layer = layer[0] if isinstance(layer, (list, tuple)) else layer
+        kc, vc, group = cache.layer_kv(kv_layer)
+        meta = ctx.kv[group]
+        bias = self.w.get("in.bias")
+        if s.conv_taps:
+            qkv = ctx.ws.take("attention.conv", (nt, self.qkv_width), self.dtype)
+            kernels.causal_conv(proj, 0, self.qkv_width, self.w["conv.weight"], qkv,
+                                cache.layer_state(layer[1]) if s.conv_taps > 1 else None, ctx.cu_q, ctx.slots,
+                                ctx.ws.take("conv.tok_seq", (nt,), torch.int32), bias_in=bias)
+            bias = None
+        else:
+            qkv = proj[:, :self.qkv_width]
+        angles = self.rotary.angles(ctx) if self.rotary is not None else None
+        kernels.qk_rotate_store(qkv, self.nq, self.nkv, self.dk, self.dv, s.own_kv, bias, angles, s.rot_dims,
+                                s.rot_style, meta.dest if (writes_cache and s.own_kv) else None, kc, vc)
+        o = ctx.ws.take("attention.o", (nt, self.nq * self.dv), self.dtype)
+        sink = self.w["sink"] if s.sink == "learned" else s.sink
+        kernels.attention_sink(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen, self.nq, self.nkv,
+                               self.dk, self.dv, float(s.scale), s.window, s.softcap, sink,
+                               proj[:, self.qkv_width:] if s.out_gate else None)
+        return linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta"), None
+
+
+register_part("attention_sink", SinkAttention)

@@ -18,11 +18,15 @@ class PreNormBlock(Part):
         self.dtype = dtype
         self.norm1 = build_part(spec.norm1, dtype, device)
         self.mixer = build_part(spec.mixer, dtype, device)
-        self.norm2 = build_part(spec.norm2, dtype, device)
-        self.ffn = build_part(spec.ffn, dtype, device)
+        # a block without a feed-forward has the mixer's sublayer only
+        self.ffn = build_part(spec.ffn, dtype, device) if spec.ffn is not None else None
+        self.norm2 = build_part(spec.norm2, dtype, device) if spec.ffn is not None else None
 
     def children(self):
-        return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2, "ffn": self.ffn}
+        c = {"norm1": self.norm1, "mixer": self.mixer}
+        if self.ffn is not None:
+            c.update(norm2=self.norm2, ffn=self.ffn)
+        return c
 
     def cache_need(self):
         return self.mixer.cache_need()
@@ -36,7 +40,7 @@ class PreNormBlock(Part):
     def graph_safe(self) -> bool:
         """True when a step of this block is a fixed sequence of kernel launches on
         fixed buffers (no host decisions that depend on the data)."""
-        return all(getattr(p, "graph_safe", False) for p in (self.norm1, self.mixer, self.norm2, self.ffn))
+        return all(getattr(p, "graph_safe", False) for p in self.children().values())
 
     # Single-token steps of a bfloat16 engine: a few-rows product in front of a norm adds to the
     # residual stream and prepares the norm itself, and the product behind it applies the
@@ -71,6 +75,9 @@ class PreNormBlock(Part):
         else:
             with span(ctx, "norm"):
                 self.norm1.run(x, h, pending[0], pending[1])
+        if self.ffn is None:
+            with span(ctx, "mixer"):
+                return self.mixer.run(h, ctx, cache, layer, writes_cache, **kw)
         fusable = self._fusable(nt)
         if (fusable and hasattr(self.norm2, "fold") and self._offers(self.mixer, "can_fold", nt)
                 and self._offers(self.ffn, "takes_scaled", nt)):

@@ -132,10 +132,22 @@ class RoutedMLP(Part):
         if not 1 <= s.top <= s.experts or s.intermediate < 1:
             raise PartError(f"routed feed-forward: top {s.top} of {s.experts} experts of {s.intermediate}")
         form = getattr(s, "form", "mlp")
-        if form not in ("mlp", "limited_glu"):
+        if form not in ("mlp", "limited_glu", "glu"):
             raise PartError(f"routed feed-forward: unknown form {form!r}")
         self.limited = form == "limited_glu"
-        if self.limited:
+        self.glu = form == "glu"                  # act(gate) * up, no limits
+        self.two = self.limited or self.glu       # an expert's first matrix is [gate rows | up rows]
+        self.groups, self.keep_groups = int(getattr(s, "groups", 1)), int(getattr(s, "keep_groups", 1))
+        if self.groups < 1 or s.experts % self.groups or not 1 <= self.keep_groups <= self.groups or \
+                s.top > self.keep_groups * (s.experts // self.groups):
+            raise PartError(f"routed feed-forward: {s.experts} experts in {self.groups} groups of which "
+                            f"{self.keep_groups} stay do not hold {s.top} choices")
+        if self.glu:
+            if s.activation not in kernels._GLU_ACTS:
+                raise PartError(f"unknown expert activation {s.activation!r}")
+            if s.shared_intermediate is not None:
+                raise PartError("routed feed-forward: the glu form has no shared expert")
+        elif self.limited:
             if not s.limit > 0 or (s.shared_intermediate is not None and not s.shared_limit > 0):
                 raise PartError(f"routed feed-forward: limits must be positive, got {s.limit} / {s.shared_limit}")
         elif s.activation not in kernels._MOE_ACTS or s.activation not in kernels._ACTIVATIONS:
@@ -147,8 +159,8 @@ class RoutedMLP(Part):
 
     def params(self):
         s = self.spec
-        # limited_glu: an expert's first matrix is [gate rows | up rows]
-        first, k = ("gate_up", 2) if self.limited else ("up", 1)
+        # limited_glu, glu: an expert's first matrix is [gate rows | up rows]
+        first, k = ("gate_up", 2) if self.two else ("up", 1)
         p = {"router.weight": Param((s.experts + int(self.gated_shared), s.hidden), "matrix"),
              f"experts.{first}.weight": Param((s.experts * k * s.intermediate, s.hidden), "matrix"),
              "experts.down.weight": Param((s.experts * s.hidden, s.intermediate), "matrix")}
@@ -163,12 +175,14 @@ class RoutedMLP(Part):
         """The first product of the experts (tile_expert given) or of the shared expert with
         its activation: rows [.., n] in the engine's type."""
         s, rows = self.spec, a.shape[0]
-        k = 2 if self.limited else 1
+        k = 2 if self.two else 1
         pre = ws.take(name + ".pre", (rows, k * n), self.dtype)
         if tile_expert is not None:
-            kernels.moe_gemm(a, w, tile_expert, pre, None if self.limited else s.activation)
+            kernels.moe_gemm(a, w, tile_expert, pre, None if self.two else s.activation)
         else:
             linear(a, w, pre)
+        if self.glu:
+            return kernels.glu(pre, ws.take(name, (rows, n), self.dtype), s.activation)
         if not self.limited:
             if tile_expert is None:
                 kernels.activation(pre, pre, s.activation)
@@ -183,7 +197,8 @@ class RoutedMLP(Part):
         logits = linear(h, self.w["router.weight"], ws.take("moe.logits", (nt, E + int(self.gated_shared)), torch.float32))
         chosen = ws.take("moe.chosen", (nt, top), torch.int32)
         weight = ws.take("moe.weight", (nt, top), torch.float32)
-        kernels.moe_route(logits, E, top, chosen, weight, s.score, s.renormalize, bias=self.w.get("router.bias"))
+        kernels.moe_route(logits, E, top, chosen, weight, s.score, s.renormalize, bias=self.w.get("router.bias"),
+                          groups=self.groups, keep_groups=self.keep_groups)
         if getattr(ctx, "dump", None) is not None:
             ctx.dump("experts", chosen)
         rows = kernels.moe_max_rows(nt * top, E)
@@ -193,7 +208,7 @@ class RoutedMLP(Part):
         kernels.moe_plan(chosen, E, row_pair, tile_expert, pair_row)
         on_input = s.weight_on == "input"
         a = kernels.moe_gather(h, top, row_pair, weight if on_input else None, ws.take("moe.a", (rows, d), self.dtype))
-        first, k = ("gate_up", 2) if self.limited else ("up", 1)
+        first, k = ("gate_up", 2) if self.two else ("up", 1)
         up = self.w[f"experts.{first}.weight"].view(E, k * ff, d)
         down = self.w["experts.down.weight"].view(E, d, ff)
         if up.dtype != self.dtype:

@@ -38,6 +38,29 @@ def scaled_frequencies(dims: int, base: float, scaling=None) -> np.ndarray:
     return np.where(wavelength < original / high, f, np.where(wavelength > original / low, f / factor, blended))
 
 
+RAMP_FLOOR = 0.001      # least width of a ramp between kept and slowed frequencies
+
+
+def ramp_frequencies(dims: int, base: float, ramp) -> np.ndarray:
+    """f_j = base^(-2j/dims), j < dims/2, float64, slowed along a ramp over the pair index: with
+    ramp = (factor, original, fast, slow) and n(t) = dims * ln(original / (2 pi t)) / (2 ln base), lo =
+    max(floor(n(fast)), 0), hi = min(ceil(n(slow)), dims - 1), r_j = clamp((j - lo) / max(hi - lo,
+    RAMP_FLOOR), 0, 1): f_j <- f_j / factor * r_j + f_j * (1 - r_j)."""
+    j = np.arange(dims // 2, dtype=np.float64)
+    f = float(base) ** (-2.0 * j / dims)
+    factor, original, fast, slow = (float(v) for v in ramp)
+    if not (factor > 0 and original > 0 and fast > 0 and slow > 0 and base > 1):
+        raise PartError(f"rotary ramp: factor {factor}, original {original}, fast {fast}, slow {slow}, base {base}")
+
+    def index(turns):
+        return dims * np.log(original / (2.0 * np.pi * turns)) / (2.0 * np.log(float(base)))
+
+    lo = max(float(np.floor(index(fast))), 0.0)
+    hi = min(float(np.ceil(index(slow))), dims - 1.0)
+    r = np.clip((j - lo) / max(hi - lo, RAMP_FLOOR), 0.0, 1.0)
+    return f / factor * r + f * (1.0 - r)
+
+
 class Rotary(Part):
     graph_safe = True
 
@@ -48,10 +71,17 @@ class Rotary(Part):
             raise PartError(f"unknown rotary pairing {spec.style!r}")
         self.head_dim = spec.head_dim
         self.interleaved = spec.style == "interleaved"
-        inv = scaled_frequencies(spec.head_dim, float(spec.theta), getattr(spec, "scaling", None))
+        scaling, ramp = getattr(spec, "scaling", None), getattr(spec, "ramp", None)
+        if scaling is not None and ramp is not None:
+            raise PartError("a rotation takes one way of slowing its frequencies, not both")
+        if ramp is not None:
+            inv = ramp_frequencies(spec.head_dim, float(spec.theta), ramp)
+        else:
+            inv = scaled_frequencies(spec.head_dim, float(spec.theta), scaling)
         self.inv_freq = torch.tensor(inv.astype(np.float32), device=device)
-        scaling = getattr(spec, "scaling", None)
-        self.key = ("rope", spec.head_dim, float(spec.theta), None if scaling is None else tuple(scaling))
+        self.magnitude = float(getattr(spec, "magnitude", 1.0))
+        self.key = ("rope", spec.head_dim, float(spec.theta), None if scaling is None else tuple(scaling),
+                    None if ramp is None else tuple(ramp), self.magnitude)
 
     def angles(self, ctx):
         """(cos, sin) of every token of the step, computed once per step and shared
@@ -60,7 +90,7 @@ class Rotary(Part):
         if table is None:
             out = ctx.ws.take("rope.angles." + ".".join(str(k) for k in self.key[1:]),
                               (ctx.nt, self.head_dim // 2, 2), torch.float32)
-            table = kernels.rope_table(ctx.positions, self.inv_freq, out)
+            table = kernels.rope_table(ctx.positions, self.inv_freq, out, self.magnitude)
             ctx.shared[self.key] = table
         return table
 

@@ -235,6 +235,73 @@ class DecayLinearAttention(Part):
         return linear_delta(gated, self.w["out.weight"], ctx.ws, "decay_attention.delta"), None
 
 
+class StateSpace(Part):
+    """The selective state-space mixer with a scalar decay per head (``StateSpaceSpec``).
+
+    One product gives [z | x | B | C | dt]; ``kernels.causal_conv`` runs the convolution with bias and
+    silu over [x | B | C] (its memory is the second piece of state); ``kernels.ssm_steps`` forms step
+    sizes and decays of every (token, head) in float32; the recurrence is the kernel of
+    ``GatedLinearAttention`` with q = C, k = B, v = x, the heads of a group reading the same B and C,
+    one decay per (token, head) and the step size as a factor on the key, so state, decays and
+    readout stay float32 and tokens are walked in order; ``kernels.gated_group_norm`` adds D x, gates
+    with silu(z) and norms the parts of the row."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        s = spec
+        if min(s.num_heads, s.head_dim, s.state, s.groups, s.taps, s.norm_groups) < 1:
+            raise PartError(f"state space: {s.num_heads} heads of {s.head_dim}, state {s.state}, {s.groups} groups, "
+                            f"{s.taps} taps, {s.norm_groups} norm parts")
+        if s.num_heads % s.groups or (s.num_heads * s.head_dim) % s.norm_groups:
+            raise PartError(f"state space: {s.num_heads} heads of {s.head_dim} do not divide into {s.groups} "
+                            f"groups / {s.norm_groups} norm parts")
+        self.spec, self.dtype = s, dtype
+        self.inner = s.num_heads * s.head_dim
+        self.gn = s.groups * s.state
+        self.conv_width = self.inner + 2 * self.gn
+        self.width = self.inner + self.conv_width + s.num_heads
+
+    def params(self):
+        s = self.spec
+        H = s.num_heads
+        return {"in.weight": Param((self.width, s.hidden), "matrix"),       # z, x, B, C, dt
+                "conv.weight": Param((self.conv_width, s.taps), "vector"),
+                "conv.bias": Param((self.conv_width,), "vector"),
+                "dt_bias": Param((H,), "vector", init="zero"),
+                "A_log": Param((H,), "vector", init="zero"),
+                "D": Param((H,), "vector", init="around_one"),
+                "norm.weight": Param((self.inner,), "vector", init="around_one"),
+                "out.weight": Param((s.hidden, self.inner), "matrix")}
+
+    def cache_need(self):
+        s = self.spec
+        need = [StateNeed((s.num_heads, s.state, s.head_dim), torch.float32)]
+        if s.taps > 1:
+            need.append(StateNeed((s.taps - 1, self.conv_width), torch.float32))
+        return need
+
+    def run(self, h, ctx, cache, layer, writes_cache=True):
+        s, nt = self.spec, h.shape[0]
+        H, P, N = s.num_heads, s.head_dim, s.state
+        proj = linear(h, self.w["in.weight"], ctx.ws.take("state_space.in", (nt, self.width), self.dtype))
+        xbc = ctx.ws.take("state_space.xbc", (nt, self.conv_width), self.dtype)
+        kernels.causal_conv(proj, self.inner, self.conv_width, self.w["conv.weight"], xbc,
+                            cache.layer_state(layer[1]) if s.taps > 1 else None, ctx.cu_q, ctx.slots,
+                            ctx.ws.take("conv.tok_seq", (nt,), torch.int32), bias_out=self.w["conv.bias"],
+                            activation="silu")
+        dt = ctx.ws.take("state_space.dt", (nt, H), torch.float32)
+        decay = ctx.ws.take("state_space.decay", (nt, H), torch.float32)
+        kernels.ssm_steps(proj, self.inner + self.conv_width, H, self.w["dt_bias"], self.w["A_log"], dt, decay)
+        o = kernels.ssm_recurrent(xbc, 0, self.inner, self.inner + self.gn, H, s.groups, N, P, decay, dt,
+                                  cache.layer_state(layer[0]), ctx.cu_q, ctx.slots,
+                                  ctx.ws.take("state_space.o", (kernels.gla_row_parts(N), nt, H, P), torch.float32))
+        y = kernels.gated_group_norm(o.view(o.shape[0], nt, self.inner), proj, 0, self.w["norm.weight"], float(s.eps),
+                                     s.norm_groups, ctx.ws.take("state_space.y", (nt, self.inner), self.dtype),
+                                     x=xbc, x_off=0, skip=self.w["D"], head_dim=P)
+        return linear_delta(y, self.w["out.weight"], ctx.ws, "state_space.delta"), None
+
+
+register_part("state_space", StateSpace)
 register_part("diagonal_recurrence", DiagonalRecurrence)
 register_part("decay_linear_attention", DecayLinearAttention)
 register_part("bonus_recurrence", BonusRecurrence)
