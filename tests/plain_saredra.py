@@ -230,8 +230,8 @@ def state_space(h, w, p, m, eps):
 
 
 def parallel_mixer(h, w, p, m, eps, positions):
-    return m["left_scale"] * conv_attention(h, w, p + "left.", m["left"], positions) + \
-        m["right_scale"] * state_space(h, w, p + "right.", m["right"], eps)
+    return m.get("left_scale", 1.0) * conv_attention(h, w, p + "left.", m["left"], positions) + \
+        m.get("right_scale", 1.0) * state_space(h, w, p + "right.", m["right"], eps)
 
 
 def dense_ff(h, w, p):
@@ -261,11 +261,28 @@ def route(s, top, group_count=1, group_keep=1):
     return np.argsort(-masked, kind="stable")[:top]
 
 
+def close_call(s, forced, top, group_count=1, group_keep=1, slack=0.0):
+    """Whether ``forced`` is what routing could choose from scores moved by at most ``slack``: its
+    groups reach the weakest kept group's score within the slack, and among the experts of the
+    groups then allowed each of its experts reaches the weakest chosen score within the slack."""
+    E = s.shape[0]
+    size = E // group_count
+    mine = sorted({int(e) // size for e in forced})
+    if len(set(int(e) for e in forced)) != top or len(mine) > group_keep:
+        return False
+    best = s.reshape(group_count, size).max(axis=1)
+    if np.any(best[mine] < np.sort(best)[::-1][group_keep - 1] - slack):
+        return False
+    others = [int(g) for g in np.argsort(-best, kind="stable") if int(g) not in mine]
+    allowed = np.concatenate([np.arange(g * size, (g + 1) * size) for g in mine + others[:group_keep - len(mine)]])
+    return bool(np.all(s[np.asarray(forced, dtype=np.int64)] >= np.sort(s[allowed])[::-1][top - 1] - slack))
+
+
 def moe(h, w, p, m, forced=None, slack=0.0):
     """Routed feed-forward: the chosen experts' results weighted by their scores (softmax over all
     experts, not renormalised). ``forced`` [T, top]: experts to use instead of the own choice,
-    accepted only where each differs from the own choice by a close call (scores within
-    ``slack``). Returns (result, chosen [T, top])."""
+    accepted only where they differ from it by a close call (``close_call`` with ``slack``).
+    Returns (result, chosen [T, top])."""
     r = m["router"]
     E, top = r["experts"], r["top"]
     gc = (r.get("groups") or {}).get("count", 1)
@@ -277,13 +294,10 @@ def moe(h, w, p, m, forced=None, slack=0.0):
     for t in range(T):
         mine = route(s[t], top, gc, gk)
         if forced is not None and set(int(e) for e in forced[t]) != set(int(e) for e in mine):
-            theirs = np.asarray(forced[t], dtype=np.int64)
-            worst_mine = min(s[t, e] for e in mine)
-            for e in theirs:
-                if e not in mine and not s[t, e] >= worst_mine - slack:
-                    raise AssertionError(f"token {t}: expert {e} (score {s[t, e]}) is no close call "
-                                         f"against {mine} ({s[t, mine]})")
-            mine = theirs
+            if not close_call(s[t], forced[t], top, gc, gk, slack):
+                raise AssertionError(f"token {t}: experts {list(forced[t])} are no close call against "
+                                     f"{list(mine)} (scores {s[t]})")
+            mine = np.asarray(forced[t], dtype=np.int64)
         chosen[t] = mine
         for e in mine:
             q = f"{p}e{int(e)}."

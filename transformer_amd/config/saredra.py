@@ -299,7 +299,7 @@ class SaredraConfig:
         rot = a.rot
         return SinkAttentionSpec(
             hidden=self.width, num_heads=a.heads, num_kv_heads=a.kv_heads, key_dim=a.dim, value_dim=a.vdim,
-            scale=a.scale, softcap=a.softcap, window=a.window, cache_window=cache_window,
+            scale=a.scale, softcap=a.softcap, window=a.window, cache_window=0 if cache_window is None else cache_window,
             sink="learned" if left else "unit", rot_dims=rot.dims if rot else 0, rot_base=rot.base if rot else 10000.0,
             rot_style="interleaved", rot_ramp=rot.scaling if rot else None, rot_magnitude=rot.magnitude() if rot else 1.0,
             qkv_bias=left, conv_taps=a.conv, out_gate=not left, own_kv=a.kv_from is None)

@@ -475,7 +475,7 @@ class SinkAttentionSpec:
     heads are multiplied by sigmoid(Wg h) before the output projection. own_kv False: no key and value
     projections; the layer reads what the layer whose cache it borrows stored (its schedule entry
     names it). cache_window: the window the cache layer is kept for (the widest of the layers that
-    read it; None: everything)."""
+    read it; 0: everything; None: the layer's own window)."""
     hidden: int
     num_heads: int
     num_kv_heads: int

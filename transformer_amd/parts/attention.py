@@ -270,7 +270,8 @@ class SinkAttention(Part):
             raise PartError(f"{s.rot_dims} rotated coordinates ({s.rot_style!r}) do not fit heads of {s.key_dim}")
         if s.window is not None and s.window < 1:
             raise PartError(f"attention window must be >= 1, got {s.window}")
-        if s.cache_window is not None and (s.window is None or s.cache_window < s.window):
+        if s.cache_window is not None and (s.cache_window < 0 or
+                                           (s.cache_window > 0 and (s.window is None or s.cache_window < s.window))):
             raise PartError(f"a cache kept for {s.cache_window} tokens does not serve a window of {s.window}")
         if s.sink not in (None, "unit", "learned"):
             raise PartError(f"unknown sink {s.sink!r}")
@@ -302,7 +303,8 @@ class SinkAttention(Part):
 
     def cache_need(self):
         s = self.spec
-        window = s.window if s.cache_window is None else s.cache_window
+        # cache_window None: the layer's own window; 0: every token is kept; else that many
+        window = s.window if s.cache_window is None else (s.cache_window or None)
         kv = KVNeed(self.nkv, self.dk, window, self.dv)
         if s.conv_taps > 1:
             from ..cache.storage import StateNeed
