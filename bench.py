@@ -255,6 +255,55 @@ def luduvik_shapes():
             "w4096": shape(4096, 32, 8, 32, 64, 6, 1408, 2816, 14336, 32000)}
 
 
+def saredra_shapes():
+    """Layer sizes that resemble real models' (random weights): Saredra models whose layers are
+    all attention or all parallel (each with the routed feed-forward), the mixed order with a
+    layer that reads another's keys and values, and the closest layers of the other decoders at
+    the same width and heads: the Luduvik decoder's parallel layer (softmax attention beside a
+    matrix-state recurrence, with routed experts of the same sizes), the Vametar decoder's
+    attention and its gated linear attention, and the Llama layer."""
+    def shape(width, heads, kv, ssm_heads, experts, top, eff, ff, vocab):
+        moe = {"kind": "moe", "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}},
+               "expert": {"ff": eff}}
+        soft = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0,
+                "mask": {"size": 1024}}
+        att = {"type": "attention", "mixer": {**soft, "rot": {"base": 500000.0, "dims": 64}}, "mlp": moe}
+        reader = {"type": "attention", "mixer": {**att["mixer"], "kv_from": 0}, "mlp": moe}
+        par = {"type": "parallel", "mlp": moe, "mixer": {
+            "left": {**soft, "conv": 4, "rot": {"base": 500000.0, "dims": 64,
+                                                 "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+            "left_scale": 1.0, "right_scale": 1.0,
+            "right": {"heads": ssm_heads, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}}}
+        base = {"architecture": "Saredra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}}
+        kinds = {"attention": [att] * 4, "parallel": [par] * 4, "mixed": [att, par, reader, att]}
+        vam = {"architecture": "Vametar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
+               "logit_scale": 2.0, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}}
+        dense = {"kind": "dense", "ff": ff}
+        lmoe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": eff, "limit": 7.0}}
+        lin = ssm_heads // 2
+        near = {
+            "luduvik_parallel": ("Luduvik", {"architecture": "Luduvik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+                                             "layers": [{"type": "parallel", "mlp": lmoe, "mixer": {
+                                                 "left": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                                          "rot": {"base": 500000.0, "dims": 64}},
+                                                 "right": {"heads": lin, "dim": 128, "vdim": 128,
+                                                           "decay": [1.0 - 2.0 ** -(5.0 + 4.0 * i / lin) for i in range(lin)]}}}] * 4}),
+            "vametar_attention": ("Vametar", {**vam, "layers": [{"type": "attention", "mlp": dense, "mixer": {
+                "heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                "rot": {"base": 500000.0, "dims": 64}}}] * 4}),
+            "vametar_gla": ("Vametar", {**vam, "layers": [{"type": "gla", "mlp": dense, "mixer": {
+                "heads": lin, "dim": 128, "vdim": 128, "tau": 16.0, "rank": 16}}] * 4}),
+            "llama": ("llama", {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": width,
+                                "num_attention_heads": heads, "num_key_value_heads": kv, "head_dim": 128,
+                                "intermediate_size": ff, "vocab_size": vocab, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+                                "tie_word_embeddings": False, "max_position_embeddings": 1 << 20, "rope_scaling": None,
+                                "num_hidden_layers": 4}),
+        }
+        return base, kinds, near
+    return {"w2048": shape(2048, 16, 4, 64, 32, 4, 1024, 8192, 32000),
+            "w4096": shape(4096, 32, 8, 128, 64, 6, 1408, 14336, 32000)}
+
+
 def _routed_parts(model):
     return [b.ffn for b in model.blocks if getattr(getattr(b, "ffn", None), "spec", None) is not None
             and getattr(b.ffn.spec, "kind", "") == "routed_mlp"]
@@ -262,7 +311,7 @@ def _routed_parts(model):
 
 def _expert_entries(sp):
     """Matrix entries of one routed expert: up and down, and a gate matrix where it has one."""
-    return (3 if getattr(sp, "form", "mlp") == "limited_glu" else 2) * sp.hidden * sp.intermediate
+    return (3 if getattr(sp, "form", "mlp") in ("limited_glu", "glu") else 2) * sp.hidden * sp.intermediate
 
 
 def _leaf_mixers(m):
@@ -423,6 +472,42 @@ def bench_luduvik(a):
     return 0
 
 
+def bench_saredra(a):
+    """Prefill and decode throughput of Saredra models whose layers are all attention, all
+    parallel, and the mixed order, beside the closest layers of the other decoders at the same
+    width. One JSON line of its own; the default workload is untouched."""
+    import torch
+    import transformer_amd as ta
+    dkey = "bf16" if a.dtype == "bfloat16" else "fp32"
+    layers = a.layers or 4
+    out = {"design": "saredra", "dtype": dkey, "layers": layers, "batch": a.batch,
+           "prefill_tokens": a.prefill_tokens, "data": "synthetic", "sizes": {}}
+
+    def fit(lay):
+        return (list(lay) * (-(-layers // len(lay))))[:layers]
+
+    for size, (base, kinds, near) in saredra_shapes().items():
+        if a.design_size and size not in a.design_size.split(","):
+            continue
+        cases = [(n, arch, c) for n, (arch, c) in near.items()] + \
+                [(n, "Saredra", {**base, "layers": lay}) for n, lay in kinds.items()]
+        if a.design_case:
+            cases = [c for c in cases if c[0] in a.design_case.split(",")]
+        rows = {}
+        for name, arch, cfg in cases:
+            if arch == "llama":
+                model = ta.random_model(ta.LlamaConfig.from_dict({**cfg, "num_hidden_layers": layers}), seed=0, dtype=a.dtype)
+            else:
+                model = ta.random_model({**cfg, "layers": fit(cfg["layers"])}, seed=0, dtype=a.dtype, architecture=arch)
+            rows[name] = _design_row(model, a, dkey)
+            del model
+            torch.cuda.empty_cache()
+            print(f"[bench] {size} {name}: {rows[name]}", file=sys.stderr, flush=True)
+        out["sizes"][size] = rows
+    print(json.dumps(out))
+    return 0
+
+
 def bench_design(a):
     """Prefill and decode throughput of Vametar models whose layers are all of one kind, and
     of the mixed order, beside the Llama decoder with layers of the same width, heads and
@@ -506,16 +591,18 @@ def main():
                     help="tokens of the prompt whose step is timed (the line's \"prefill\")")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
-    ap.add_argument("--design", default=None, choices=["vametar", "kunitar", "luduvik"],
+    ap.add_argument("--design", default=None, choices=["vametar", "kunitar", "luduvik", "saredra"],
                     help="instead of the default workload: prefill and decode of this design at a few "
                          "layer sizes, beside the Llama decoder at the same sizes (a line of its own)")
     ap.add_argument("--design-size", default=None, help="with --design: only these sizes (w2048,w4096)")
-    ap.add_argument("--design-case", default=None, help="with --design kunitar or luduvik: only these rows (llama,latent,...)")
+    ap.add_argument("--design-case", default=None, help="with --design kunitar, luduvik or saredra: only these rows (llama,latent,...)")
     a = ap.parse_args()
     if a.design == "kunitar" and a.gpus == 1:
         return bench_kunitar(a)
     if a.design == "luduvik" and a.gpus == 1:
         return bench_luduvik(a)
+    if a.design == "saredra" and a.gpus == 1:
+        return bench_saredra(a)
     if a.design and a.gpus == 1:
         return bench_design(a)
     if a.gpus != 1:

@@ -272,3 +272,17 @@ def test_plain_model_is_causal_and_adds_its_sublayers_in_turn():
     h = P.rms_norm(layers[0], w["l1.norm1"], eps)          # a layer without a feed-forward adds its mixer alone
     np.testing.assert_allclose(layers[1], layers[0] + P.parallel_mixer(h, w, "l1.mix.", c["layers"][1]["mixer"], eps, np.arange(3)),
                                atol=1e-12)
+
+
+def test_bench_shapes_of_the_design_option_are_valid_models():
+    import bench
+    import transformer_amd as ta
+    for size, (base, kinds, near) in bench.saredra_shapes().items():
+        for kind, layers in kinds.items():
+            cfg = ta.SaredraConfig.from_dict({**base, "layers": layers})
+            spec = cfg.model_spec()
+            assert len(spec.blocks) == len(layers) and spec.hidden == base["width"], (size, kind)
+        assert [r.cache_of for r in ta.SaredraConfig.from_dict({**base, "layers": kinds["mixed"]}).model_spec().schedule] == \
+            [None, None, 0, None]
+        for arch, cfg_dict in near.values():
+            assert ta.get_architecture(arch).config_from_dict(cfg_dict).model_spec().hidden == base["width"]

@@ -230,6 +230,67 @@ def test_capped_sunk_softmax_pieces(dtype, geom):
     _close(np.concatenate(got), want, dtype, scale=1.5)
 
 
+@pytest.mark.parametrize("exact", [True, False])
+@pytest.mark.parametrize("geom", [(8, 2, 128, 64, 64, (2.0, 512, 16.0, 1.0), 100, 50.0, "unit", True),
+                                  (4, 4, 32, 32, 0, None, None, None, "learned", False),
+                                  (16, 4, 64, 64, 32, None, 129, 30.0, "learned", True),
+                                  (2, 1, 96, 40, 96, (3.0, 40, 6.0, 2.0), 64, 3.0, None, True),
+                                  (6, 1, 160, 8, 10, None, 1, 9.0, "unit", False),
+                                  (64, 2, 64, 64, 64, None, 200, 20.0, "learned", True)])
+def test_capped_sunk_softmax_on_matrix_cores(geom, exact):
+    """The same on the matrix-core kernels (bfloat16, value rows of the cache as wide as the keys, the
+    rest zero): prompts through the kernel that reads pages directly and the one that shares them
+    through LDS, single tokens through the kernel of four waves and the merge, with a page table
+    wider than needed; with the weights kept at 32 bits the result is as close as the vector kernel's."""
+    from transformer_amd import kernels as K
+    from transformer_amd.kernels import PAGE
+    H, G, dk, dv, rot, scaling, window, cap, sink, gated = geom
+    dtype = "bfloat16"
+    rng = np.random.default_rng(H * 7 + dk)
+    T, scale, base = 600, 0.21 * (32 / dk) ** 0.5, 500.0
+    cols = (H + G) * dk + G * dv
+    rows = _bf(rng.standard_normal((T, cols)), dtype)
+    gate = _bf(rng.standard_normal((T, H * dv + 8)), dtype)
+    rotd, mag = None, 1.0
+    if rot:
+        rotd = {"dims": rot, "base": base}
+        if scaling:
+            rotd["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+        mag = P.rotation_frequencies(rotd)[1]
+    sinks = rng.standard_normal(H) * 2.0
+    q = P.rotate_pairs(rows[:, :H * dk].reshape(T, H, dk), np.arange(T), rotd)
+    k = P.rotate_pairs(rows[:, H * dk:(H + G) * dk].reshape(T, G, dk), np.arange(T), rotd)
+    v = rows[:, (H + G) * dk:].reshape(T, G, dv)
+    want = P.windowed_softmax_attention(_bf(q, dtype), _bf(k, dtype), v, scale, cap, window,
+                                        None if sink is None else np.zeros(H) if sink == "unit" else sinks)
+    want = want.reshape(T, H * dv)
+    if gated:
+        want = want * P.sigmoid(gate[:, :H * dv])
+    kc = torch.full((12, G, PAGE, dk), float("nan"), dtype=TD[dtype], device=DEV)
+    vc = torch.full((12, G, dk, PAGE), float("nan"), dtype=TD[dtype], device=DEV)
+    pages = np.array([7, 2, 5, 11, 0, 9, 4, 1, 3, 10, 0, 0])              # ten pages of a table of twelve
+    inv = _t(P.rotation_frequencies(rotd)[0]) if rot else None
+    got, at = [], 0
+    for n, lds in ((70, 0), (300, 1), (1, None), (1, 0), (28, 0), (1, None), (199, 0)):
+        p = np.arange(at, at + n)
+        qkv = _t(rows[p], TD[dtype])
+        angles = K.rope_table(_t(p, torch.int32), inv, torch.empty(n, rot // 2, 2, device=DEV), mag) if rot else None
+        dest = _t(pages[p // PAGE] * PAGE + p % PAGE, torch.int32)
+        K.qk_rotate_store(qkv, H, G, dk, dv, True, None, angles, rot, "interleaved", dest, kc, vc)
+        o = torch.empty(n, H * dk, dtype=TD[dtype], device=DEV)
+        args = (qkv, o, kc, vc, _t([pages], torch.int32), _t([0, n], torch.int32), _t([at], torch.int32))
+        opts = (H, G, dk, scale, window, cap, _t(sinks) if sink == "learned" else sink, _t(gate[p], TD[dtype]) if gated else None, dv)
+        if lds is None:
+            K.attention_keys_sink(*args, at + 1, *opts, exact=exact)
+        else:
+            K.attention_rows_sink(*args, n, *opts, exact=exact, through_lds=lds)
+        o = _np(o).reshape(n, H, dk)
+        assert np.all(o[:, :, dv:] == 0.0)                                   # the padding of the values stays zero
+        got.append(o[:, :, :dv].reshape(n, H * dv))
+        at += n
+    _close(np.concatenate(got), want, dtype, scale=1.5 if exact else 3.0)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("where", ["prompt", "decode"])
 @pytest.mark.parametrize("mark,window", [(0, None), (3, None), (63, None), (64, None), (127, None), (128, None), (298, None),

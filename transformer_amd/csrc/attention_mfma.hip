@@ -58,6 +58,38 @@ union Frag8 {
 
 __device__ __forceinline__ uint32_t pack2(float a, float b) { return f32x2_to_bf16x2_bits(a, b); }
 
+// Options of a capped, sunk and gated softmax; all zero: the plain one.
+//   cap_k, cap_r: score <- cap_r * tanh(score * cap_k'), with the raw score q.k before the scale, cap_k =
+//     2 log2(e) * scale / cap and cap_r = cap / scale, so that the capped number takes the place
+//     of the raw score everywhere after (cap_k 0: not capped)
+//   exact: the softmax weights enter the second product as three bfloat16 pieces whose sum is the
+//     float32 weight, so only keys and values are rounded to 16 bits
+//   sink_mode 1: the denominator holds one more term exp(0); 2: exp(sink[head])
+//   gate: rows [token][gate_stride] whose sigmoid multiplies the first gate_dv columns of every head
+struct AttnExtra {
+  float cap_k, cap_r;
+  int exact, sink_mode;
+  const float* sink;
+  const bf16_t* gate;
+  int gate_stride, gate_dv;
+};
+
+__device__ __forceinline__ float capped_score(float s, float cap_k, float cap_r) {
+  const float e = __builtin_amdgcn_exp2f(s * cap_k);            // exp(2 x): tanh x = 1 - 2 / (e + 1)
+  return cap_r * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
+}
+// what the sink adds to a row's sum, relative to the reference m_use (log2 domain)
+__device__ __forceinline__ float sink_term(const AttnExtra& x, int head, float m_use) {
+  if (x.sink_mode == 0) return 0.f;
+  const float sv = x.sink_mode == 2 ? x.sink[head] * 1.4426950408889634f : 0.f;
+  return __builtin_amdgcn_exp2f(sv - m_use);
+}
+__device__ __forceinline__ float gate_factor(const AttnExtra& x, size_t token, int head, int d) {
+  if (x.gate == nullptr || d >= x.gate_dv) return 1.f;
+  const float g = to_f32(x.gate[token * x.gate_stride + (size_t)head * x.gate_dv + d]);
+  return 1.0f / (1.0f + __expf(-g));
+}
+
 // Maximum and sum over the lanes 16 or 32 apart, by the lane-swap instructions of gfx950 (one
 // vector operation each; a shuffle goes through the LDS crossbar and costs over a hundred
 // cycles in the middle of a chain). After the swap one register holds the values of the even
@@ -104,11 +136,11 @@ struct WaveState {
 // KSTR / VSTR: elements between rows of the K tile / of the V^T tile (a page in global
 // memory, or a padded copy in LDS). ZERO_TAIL: unwritten keys of the V^T tile still
 // have to be read as zero (the LDS copy is cleaned when it is stored).
-template <int DH, int KSTR, int VSTR, bool ZERO_TAIL, bool EARLY_V = false>
+template <int DH, int KSTR, int VSTR, bool ZERO_TAIL, bool EARLY_V = false, bool XTRA = false>
 __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __restrict__ kp,
                                           const bf16_t* __restrict__ vp, int key0, int my_start,
                                           int my_end, int kv_len, bool all_visible,
-                                          float scale_log2, int j, int h) {
+                                          float scale_log2, int j, int h, const AttnExtra& x = AttnExtra{}) {
   constexpr int KS = DH / 16, MT = DH / 32;
   // EARLY_V: the value operands are requested before the first product, so that a wave
   // that has only a page or two to do waits for memory once, not twice
@@ -135,6 +167,12 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
       acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, w.qf[ks].v, acc, 0, 0, 0);
     }
     s[sub] = acc;
+  }
+  if (XTRA && x.cap_k != 0.f) {    // the same for every lane
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[sub][r] = capped_score(s[sub][r], x.cap_k, x.cap_r);
   }
   // softmax of the lane's row over this page. Scores stay raw; the running maximum is
   // kept in the log2 domain (raw * scale * log2 e), so an exponent is one fma + exp2.
@@ -178,14 +216,24 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
       for (int r = 0; r < 16; ++r) w.o[mt][r] *= alpha;
   }
 
+  const bool partial = ZERO_TAIL && key0 + TA_PAGE > kv_len;   // unwritten keys hold anything: read them as 0
+  // exact: three passes, each with the bfloat16 rounding of what the passes before left of the weights
+  const int pieces = (XTRA && x.exact) ? 3 : 1;
+#pragma unroll 1
+  for (int piece = 0; piece < pieces; ++piece) {
   Frag pb[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-      pb[t].w[e] = pack2(s[t / 2][8 * (t % 2) + 2 * e], s[t / 2][8 * (t % 2) + 2 * e + 1]);
-
-  const bool partial = ZERO_TAIL && key0 + TA_PAGE > kv_len;   // unwritten keys hold anything: read them as 0
+    for (int e = 0; e < 4; ++e) {
+      const int i0 = 8 * (t % 2) + 2 * e;
+      const uint32_t two = pack2(s[t / 2][i0], s[t / 2][i0 + 1]);
+      pb[t].w[e] = two;
+      if (XTRA && x.exact) {
+        s[t / 2][i0] -= __uint_as_float(two << 16);
+        s[t / 2][i0 + 1] -= __uint_as_float(two & 0xffff0000u);
+      }
+    }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const bf16_t* vrow = vp + (mt * 32 + j) * VSTR + 4 * h;
@@ -205,6 +253,7 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
       }
       w.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pb[t].v, w.o[mt], 0, 0, 0);
     }
+  }
   }
 }
 
@@ -226,13 +275,39 @@ __device__ __forceinline__ void wave_init(WaveState<DH>& w, const bf16_t* __rest
   w.l = 0.f;
 }
 
+// A finished row: the sink's share of the denominator, the division, the heads' gate, one rounding.
+template <int DH, bool XTRA>
+__device__ __forceinline__ void rows_write(const WaveState<DH>& w, bf16_t* __restrict__ o, size_t token, int head,
+                                           int h, const AttnExtra& x) {
+  const float m_use = (w.m == -INFINITY) ? 0.f : w.m;
+  const float l = XTRA ? w.l + sink_term(x, head, m_use) : w.l;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+#pragma unroll
+  for (int mt = 0; mt < DH / 32; ++mt)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      const int d = 32 * mt + 8 * g4 + 4 * h;
+      float r[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = w.o[mt][4 * g4 + e] * inv;
+      if (XTRA && x.gate != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] *= gate_factor(x, token, head, d + e);
+      }
+      uint2 v;
+      v.x = pack2(r[0], r[1]);
+      v.y = pack2(r[2], r[3]);
+      *reinterpret_cast<uint2*>(o + d) = v;
+    }
+}
+
 // ------------------------------------------------------------------ rows: prompts
-template <int DH>
+template <int DH, bool XTRA = false>
 __global__ __launch_bounds__(256) void attn_rows_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
-    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window) {
+    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window, AttnExtra x) {
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int j = lane % 32, h = lane / 32;
   const int b = blockIdx.z, kvh = blockIdx.y;
@@ -276,22 +351,9 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(
     const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bool all_visible = all_rows && key0 + TA_PAGE <= tile_min_end && key0 >= tile_max_start;
-    wave_page<DH, DH, TA_PAGE, true>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
+    wave_page<DH, DH, TA_PAGE, true, false, XTRA>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h, x);
   }
-  if (row_ok) {
-    const float inv = w.l > 0.f ? 1.0f / w.l : 0.f;
-    bf16_t* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * DH;
-#pragma unroll
-    for (int mt = 0; mt < DH / 32; ++mt)
-#pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const int d = 32 * mt + 8 * g4 + 4 * h;
-        uint2 v;
-        v.x = pack2(w.o[mt][4 * g4 + 0] * inv, w.o[mt][4 * g4 + 1] * inv);
-        v.y = pack2(w.o[mt][4 * g4 + 2] * inv, w.o[mt][4 * g4 + 3] * inv);
-        *reinterpret_cast<uint2*>(o + d) = v;
-      }
-  }
+  if (row_ok) rows_write<DH, XTRA>(w, out + (size_t)(q0 + qi) * out_stride + (size_t)head * DH, (size_t)(q0 + qi), head, h, x);
 }
 
 // ------------------------------------------------------------------ rows through LDS
@@ -300,12 +362,12 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(
 // crosses the L2 once per 128 rows. The next page travels global -> registers while the
 // current one is multiplied, and registers -> LDS between two barriers. Rows are padded
 // (K by 16 bytes, V^T by 8) so that the operand reads of a wave spread over all banks.
-template <int DH>
+template <int DH, bool XTRA = false>
 __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
-    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window, int pair) {
+    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window, int pair, AttnExtra x) {
   constexpr int KSTR = DH + 8, VSTR = TA_PAGE + 4;
   constexpr int PER = TA_PAGE * DH / 8 / 256;          // 16-byte pieces of a page per thread
   // two page buffers: the next page is stored while the current one is multiplied
@@ -421,26 +483,13 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
     }
     if (key0 < tile_end && key0 + TA_PAGE > tile_start) {
       const bool all_visible = all_rows && key0 + TA_PAGE <= tile_min_end && key0 >= tile_max_start;
-      wave_page<DH, KSTR, VSTR, false>(w, Ks[pg & 1], Vs[pg & 1], key0, my_start, my_end, kv_len, all_visible,
-                                       scale_log2, j, h);
+      wave_page<DH, KSTR, VSTR, false, false, XTRA>(w, Ks[pg & 1], Vs[pg & 1], key0, my_start, my_end, kv_len, all_visible,
+                                       scale_log2, j, h, x);
     }
   }
 #undef STORE_PAGE
 #undef FETCH_PAGE
-  if (row_ok) {
-    const float inv = w.l > 0.f ? 1.0f / w.l : 0.f;
-    bf16_t* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * DH;
-#pragma unroll
-    for (int mt = 0; mt < DH / 32; ++mt)
-#pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const int d = 32 * mt + 8 * g4 + 4 * h;
-        uint2 v;
-        v.x = pack2(w.o[mt][4 * g4 + 0] * inv, w.o[mt][4 * g4 + 1] * inv);
-        v.y = pack2(w.o[mt][4 * g4 + 2] * inv, w.o[mt][4 * g4 + 3] * inv);
-        *reinterpret_cast<uint2*>(o + d) = v;
-      }
-  }
+  if (row_ok) rows_write<DH, XTRA>(w, out + (size_t)(q0 + qi) * out_stride + (size_t)head * DH, (size_t)(q0 + qi), head, h, x);
   }
 }
 
@@ -880,14 +929,15 @@ __global__ __launch_bounds__(256, 2) void attn_rows_halves_kernel(
 // rotates and stores the new key and stores the new value, then waits at a barrier:
 // that page is read by this workgroup only, and a barrier makes a workgroup's global
 // writes visible to itself.
-template <int DH, int WAVES>
+template <int DH, int WAVES, bool XTRA = false>
 __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, const float* __restrict__ bias,
     const float2* __restrict__ cs, int style, const int* __restrict__ dest,
     bf16_t* __restrict__ out, int out_stride, bf16_t* __restrict__ kcache,
     bf16_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window,
-    const int* __restrict__ units, const int* __restrict__ seq_units, float* __restrict__ partial) {
+    const int* __restrict__ units, const int* __restrict__ seq_units, float* __restrict__ partial,
+    AttnExtra x = AttnExtra{}) {
   extern __shared__ float lds[];
   constexpr int KS = DH / 16, HALF = DH / 2;
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
@@ -1029,7 +1079,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
     const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bool all_visible = key0 + TA_PAGE <= kv_len && key0 >= vis_start;   // rows beyond nrows are never written
-    wave_page<DH, DH, TA_PAGE, true, true>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
+    wave_page<DH, DH, TA_PAGE, true, true, XTRA>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h, x);
   }
 
   // ---- merge the waves: lds = ml[WAVES][32][2] then o[WAVES][nrows][DH]
@@ -1062,8 +1112,10 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
     }
     const int hd = kvh * group + hg0 + r;
     if (splits == 1) {
+      if (XTRA) ll += sink_term(x, hd, m_use);
       const float inv = ll > 0.f ? 1.0f / ll : 0.f;
-      out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
+      const float gf = XTRA ? gate_factor(x, (size_t)b, hd, d) : 1.f;
+      out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(XTRA ? acc * inv * gf : acc * inv);
     } else {
       float* pr = partial + ((size_t)blockIdx.y * nh + hd) * (DH + 2);
       pr[d] = acc;
@@ -1735,9 +1787,10 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
 // one unit has its rows already. The partial rows of up to eight units are asked for at once
 // (their maxima, sums and this thread's element), so that the kernel is two trips to memory
 // behind its launch and not one per pass over the units.
-template <int DH>
+template <int DH, bool XTRA = false>
 __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
-                                  int out_stride, int nh, const int* __restrict__ seq_units) {
+                                  int out_stride, int nh, const int* __restrict__ seq_units,
+                                  AttnExtra x = AttnExtra{}) {
   const int hd = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const int first = seq_units[2 * b], splits = seq_units[2 * b + 1];
   if (splits <= 1) return;
@@ -1771,8 +1824,10 @@ __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __r
     }
     mm = gm;
   }
+  if (XTRA) ll += sink_term(x, hd, (mm == -INFINITY) ? 0.f : mm);
   const float inv = ll > 0.f ? 1.0f / ll : 0.f;
-  out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
+  const float gf = XTRA ? gate_factor(x, (size_t)b, hd, d) : 1.f;
+  out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(XTRA ? acc * inv * gf : acc * inv);
 }
 
 // ------------------------------------------------------------------ host side
@@ -1805,11 +1860,28 @@ static int check_common(const char* what, int batch, int nh, int nkv, int dh, in
 static const float LOG2E = 1.4426950408889634f;
 
 // Prompts (any mix of lengths, also single tokens). Same arguments as ta_attention_generic.
-extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_stride, void* out,
-                                      int out_stride, const void* kcache, const void* vcache,
-                                      const int* block_table, int max_blocks, const int* cu_q,
-                                      const int* pos0, int batch, int max_qlen, int nh, int nkv,
-                                      int dh, float scale, int window, int use_lds) {
+static int make_extra(const char* what, AttnExtra* x, int nh, int dh, float scale, float softcap, int exact,
+                      int sink_mode, const float* sink, const void* gate, int gate_stride, int gate_dv) {
+  TA_REQUIRE(softcap >= 0.f && scale > 0.f, "%s: cap %f / scale %f", what, softcap, scale);
+  TA_REQUIRE(sink_mode >= 0 && sink_mode <= 2 && (sink_mode != 2 || sink != nullptr), "%s: sink mode %d", what, sink_mode);
+  TA_REQUIRE(gate == nullptr || (gate_dv >= 1 && gate_dv <= dh && gate_stride >= nh * gate_dv),
+             "%s: gate rows of %d for %d heads of %d", what, gate_stride, nh, gate_dv);
+  x->cap_k = softcap > 0.f ? 2.0f * 1.4426950408889634f * scale / softcap : 0.f;
+  x->cap_r = softcap > 0.f ? softcap / scale : 0.f;
+  x->exact = exact ? 1 : 0;
+  x->sink_mode = sink_mode;
+  x->sink = sink;
+  x->gate = (const bf16_t*)gate;
+  x->gate_stride = gate_stride;
+  x->gate_dv = gate_dv;
+  return 0;
+}
+
+static int attention_rows_launch(hipStream_t stream, const void* q, int q_stride, void* out,
+                                 int out_stride, const void* kcache, const void* vcache,
+                                 const int* block_table, int max_blocks, const int* cu_q,
+                                 const int* pos0, int batch, int max_qlen, int nh, int nkv,
+                                 int dh, float scale, int window, int use_lds, const AttnExtra& x, bool plain) {
   if (check_common("ta_attention_rows_bf16", batch, nh, nkv, dh, q_stride, out_stride, max_blocks, q, out)) return 1;
   TA_REQUIRE(max_qlen >= 0 && nkv <= 65535, "ta_attention_rows_bf16: bad max_qlen=%d or nkv=%d", max_qlen, nkv);
   if (batch == 0 || max_qlen == 0) return 0;
@@ -1818,6 +1890,7 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
   TA_REQUIRE(use_lds >= 0 && use_lds <= 2, "ta_attention_rows_bf16: unknown kernel %d", use_lds);
   dim3 g((unsigned)((rows + 127) / 128), nkv, batch), blk(256);
   if (use_lds == 2) {
+    TA_REQUIRE(plain, "ta_attention_rows_bf16: the kernel that overlaps by half pages takes the plain softmax only");
     TA_REQUIRE(dh <= 128, "ta_attention_rows_bf16: the kernel that overlaps by half pages takes head sizes up to 128 (%d)", dh);
     // two blocks of rows per workgroup once that still fills every CU twice (two workgroups
     // share one); 2: one block each, all on the CUs at once, see the kernel
@@ -1855,17 +1928,50 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
     // L2; with the row blocks fastest every XCD read every head's pages and they did not.
     TA_REQUIRE(g.x <= 65535, "ta_attention_rows_bf16: prompt too long for one launch");
     g = dim3(nkv, g.x, batch);
-    DISPATCH_DH(dh, (attn_rows_lds_kernel<DH><<<g, blk, 0, stream>>>(
-                        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
-                        (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
-                        scale * LOG2E, window, pair)));
+#define ROWS_LDS(X)                                                                                        \
+  DISPATCH_DH(dh, (attn_rows_lds_kernel<DH, X><<<g, blk, 0, stream>>>(                                   \
+                      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,       \
+                      (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, scale * LOG2E, \
+                      window, pair, x)))
+    if (plain) { ROWS_LDS(false); } else { ROWS_LDS(true); }
+#undef ROWS_LDS
   } else {
-    DISPATCH_DH(dh, (attn_rows_kernel<DH><<<g, blk, 0, stream>>>(
-                        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
-                        (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
-                        scale * LOG2E, window)));
+#define ROWS_DIRECT(X)                                                                                     \
+  DISPATCH_DH(dh, (attn_rows_kernel<DH, X><<<g, blk, 0, stream>>>(                                       \
+                      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,       \
+                      (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, scale * LOG2E, \
+                      window, x)))
+    if (plain) { ROWS_DIRECT(false); } else { ROWS_DIRECT(true); }
+#undef ROWS_DIRECT
   }
   return ta_check_launch("ta_attention_rows_bf16");
+}
+
+extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_stride, void* out,
+                                      int out_stride, const void* kcache, const void* vcache,
+                                      const int* block_table, int max_blocks, const int* cu_q,
+                                      const int* pos0, int batch, int max_qlen, int nh, int nkv,
+                                      int dh, float scale, int window, int use_lds) {
+  return attention_rows_launch(stream, q, q_stride, out, out_stride, kcache, vcache, block_table, max_blocks, cu_q,
+                               pos0, batch, max_qlen, nh, nkv, dh, scale, window, use_lds, AttnExtra{}, true);
+}
+
+// The same with the options of a capped, sunk and gated softmax (see AttnExtra): softcap > 0 caps the
+// scaled scores; exact: 32-bit softmax weights in the second product; sink_mode / sink; gate rows
+// [tokens][gate_stride] with gate_dv columns per head. use_lds 0 or 1.
+extern "C" int ta_attention_rows_sink_bf16(hipStream_t stream, const void* q, int q_stride, void* out,
+                                           int out_stride, const void* kcache, const void* vcache,
+                                           const int* block_table, int max_blocks, const int* cu_q,
+                                           const int* pos0, int batch, int max_qlen, int nh, int nkv,
+                                           int dh, float scale, int window, int use_lds, float softcap, int exact,
+                                           int sink_mode, const float* sink, const void* gate, int gate_stride,
+                                           int gate_dv) {
+  AttnExtra x;
+  if (make_extra("ta_attention_rows_sink_bf16", &x, nh, dh, scale, softcap, exact, sink_mode, sink, gate, gate_stride, gate_dv))
+    return 1;
+  TA_REQUIRE(use_lds == 0 || use_lds == 1, "ta_attention_rows_sink_bf16: kernels 0 and 1 take the options, not %d", use_lds);
+  return attention_rows_launch(stream, q, q_stride, out, out_stride, kcache, vcache, block_table, max_blocks, cu_q,
+                               pos0, batch, max_qlen, nh, nkv, dh, scale, window, use_lds, x, false);
 }
 
 // Floats of scratch the single-token kernels need for `n_units` units of work.
@@ -1889,13 +1995,15 @@ extern "C" long long ta_attention_keys_scratch(int n_units, int nh, int dh) {
 // Fused use: qkv = [q | k | v] raw projections; bias (float32 per column) is added, q and k
 // are rotated by cs ([batch][dh/2] (cos, sin); null: no rotation; style 0 pairs (j, j+dh/2),
 // 1 pairs (2j, 2j+1)) and the new key and value are stored at dest[b] = page * 64 + offset.
-extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q_stride,
-                                      const float* bias, const float* cs, int style,
-                                      const int* dest, void* out, int out_stride, void* kcache,
-                                      void* vcache, const int* block_table, int max_blocks,
-                                      const int* pos0, int batch, int nh, int nkv, int dh,
-                                      float scale, int window, const int* units,
-                                      const int* seq_units, int n_units, int waves, float* scratch) {
+static int attention_keys_launch(hipStream_t stream, const void* qkv, int q_stride,
+                                 const float* bias, const float* cs, int style,
+                                 const int* dest, void* out, int out_stride, void* kcache,
+                                 void* vcache, const int* block_table, int max_blocks,
+                                 const int* pos0, int batch, int nh, int nkv, int dh,
+                                 float scale, int window, const int* units,
+                                 const int* seq_units, int n_units, int waves, float* scratch,
+                                 const AttnExtra& x, bool plain) {
+  TA_REQUIRE(plain || waves == 4, "ta_attention_keys_bf16: the options of the capped softmax go with the kernel of 4 waves");
   if (check_common("ta_attention_keys_bf16", batch, nh, nkv, dh, q_stride, out_stride, max_blocks, qkv, out)) return 1;
   TA_REQUIRE(n_units >= batch && n_units <= 65535 && units != nullptr && seq_units != nullptr,
              "ta_attention_keys_bf16: %d units of work for %d sequences", n_units, batch);
@@ -1927,18 +2035,50 @@ extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q
     DISPATCH_DH(dh, (attn_keys_q16_kernel<DH><<<g, blk, 0, stream>>>(KEYS_ARGS)));
   } else if (waves == 1) {
     DISPATCH_DH(dh, (attn_keys_lds_kernel<DH><<<g, blk, 0, stream>>>(KEYS_ARGS)));
+  } else if (!plain) {           // the options: four waves take pages in turn
+    DISPATCH_DH(dh, (attn_keys_kernel<DH, 4, true><<<g, blk, lds, stream>>>(KEYS_ARGS, x)));
   } else if (waves == 8) {
-    DISPATCH_DH(dh, (attn_keys_kernel<DH, 8><<<g, blk, lds, stream>>>(KEYS_ARGS)));
+    DISPATCH_DH(dh, (attn_keys_kernel<DH, 8><<<g, blk, lds, stream>>>(KEYS_ARGS, x)));
   } else {
-    DISPATCH_DH(dh, (attn_keys_kernel<DH, 4><<<g, blk, lds, stream>>>(KEYS_ARGS)));
+    DISPATCH_DH(dh, (attn_keys_kernel<DH, 4><<<g, blk, lds, stream>>>(KEYS_ARGS, x)));
   }
 #undef KEYS_ARGS
   if (ta_check_launch("ta_attention_keys_bf16")) return 1;
   dim3 g2(nh, batch);
-  DISPATCH_DH(dh, (attn_merge_kernel<DH><<<g2, DH, 0, stream>>>(scratch, (bf16_t*)out, out_stride, nh,
-                                                               seq_units)));
+  if (plain) {
+    DISPATCH_DH(dh, (attn_merge_kernel<DH><<<g2, DH, 0, stream>>>(scratch, (bf16_t*)out, out_stride, nh, seq_units, x)));
+  } else {
+    DISPATCH_DH(dh, (attn_merge_kernel<DH, true><<<g2, DH, 0, stream>>>(scratch, (bf16_t*)out, out_stride, nh, seq_units, x)));
+  }
   return ta_check_launch("ta_attention_keys_bf16 (merge)");
-  return 0;
+}
+
+extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q_stride,
+                                      const float* bias, const float* cs, int style,
+                                      const int* dest, void* out, int out_stride, void* kcache,
+                                      void* vcache, const int* block_table, int max_blocks,
+                                      const int* pos0, int batch, int nh, int nkv, int dh,
+                                      float scale, int window, const int* units,
+                                      const int* seq_units, int n_units, int waves, float* scratch) {
+  return attention_keys_launch(stream, qkv, q_stride, bias, cs, style, dest, out, out_stride, kcache, vcache,
+                               block_table, max_blocks, pos0, batch, nh, nkv, dh, scale, window, units, seq_units,
+                               n_units, waves, scratch, AttnExtra{}, true);
+}
+
+// Single tokens with the options of a capped, sunk and gated softmax (see AttnExtra); q holds rotated
+// heads and the cache the step's keys and values. waves 4.
+extern "C" int ta_attention_keys_sink_bf16(hipStream_t stream, const void* q, int q_stride, void* out, int out_stride,
+                                           void* kcache, void* vcache, const int* block_table, int max_blocks,
+                                           const int* pos0, int batch, int nh, int nkv, int dh, float scale,
+                                           int window, const int* units, const int* seq_units, int n_units,
+                                           int waves, float* scratch, float softcap, int exact, int sink_mode,
+                                           const float* sink, const void* gate, int gate_stride, int gate_dv) {
+  AttnExtra x;
+  if (make_extra("ta_attention_keys_sink_bf16", &x, nh, dh, scale, softcap, exact, sink_mode, sink, gate, gate_stride, gate_dv))
+    return 1;
+  return attention_keys_launch(stream, q, q_stride, nullptr, nullptr, 0, nullptr, out, out_stride, kcache, vcache,
+                               block_table, max_blocks, pos0, batch, nh, nkv, dh, scale, window, units, seq_units,
+                               n_units, waves, scratch, x, false);
 }
 
 // ------------------------------------------------------------------ no allocation

@@ -322,13 +322,13 @@ extern "C" int ta_qk_prepare(hipStream_t stream, int dtype, void* qkv, int strid
 // has q only: nkv_own = 0). bias [columns] float32 or null is added first. The first `rot` coordinates
 // of every head of q and k turn by the token's angles cs [nt, rot/2] (cos, sin): style 0 pairs
 // (i, i + rot/2), style 1 pairs (2i, 2i + 1). q goes back in place; k and v go to the paged cache at
-// dest[t] (keys [pages][kv heads][PAGE][dk], values [pages][kv heads][dv][PAGE]). float32 inside, one
-// rounding of each result. One workgroup per token, a thread per pair of coordinates.
+// dest[t] (keys [pages][kv heads][PAGE][dk], values [pages][kv heads][dvs][PAGE], dvs >= dv, rows dv.. of
+// a token zero). float32 inside, one rounding of each result. One workgroup per token, a thread per pair of coordinates.
 template <typename T>
 __global__ __launch_bounds__(256) void qk_rotate_store_kernel(
     T* __restrict__ qkv, int stride, const float* __restrict__ bias, const float2* __restrict__ cs, int rot,
     int style, const int* __restrict__ dest, T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv,
-    int nkv_own, int dk, int dv) {
+    int nkv_own, int dk, int dv, int dvs) {
   const int t = blockIdx.x;
   T* row = qkv + (size_t)t * stride;
   const int nq = nh * dk, nk = nkv_own * dk, nv = nkv_own * dv;
@@ -367,14 +367,20 @@ __global__ __launch_bounds__(256) void qk_rotate_store_kernel(
       float v = to_f32(row[nq + nk + i]);
       if (bias) v += bias[nq + nk + i];
       const int g = i / dv, c = i - g * dv;
-      vcache[(((size_t)page * nkv + g) * dv + c) * TA_PAGE + off] = from_f32<T>(v);
+      vcache[(((size_t)page * nkv + g) * dvs + c) * TA_PAGE + off] = from_f32<T>(v);
+    }
+    const int pad = dvs - dv;                          // a cache whose value rows are wider holds zeros there
+    for (int i = threadIdx.x; i < nkv_own * pad; i += 256) {
+      const int g = i / pad, c = dv + (i - g * pad);
+      vcache[(((size_t)page * nkv + g) * dvs + c) * TA_PAGE + off] = from_f32<T>(0.f);
     }
   }
 }
 
 extern "C" int ta_qk_rotate_store(hipStream_t stream, int dtype, void* qkv, int stride, const float* bias,
                                   const float* cs, int rot, int style, const int* dest, void* kcache, void* vcache,
-                                  int nt, int nh, int nkv, int nkv_own, int dk, int dv) {
+                                  int nt, int nh, int nkv, int nkv_own, int dk, int dv, int dvs) {
+  TA_REQUIRE(dvs >= dv, "ta_qk_rotate_store: value rows of %d do not hold values of %d", dvs, dv);
   TA_REQUIRE(nt >= 0 && nh >= 1 && nkv >= 1 && (nkv_own == 0 || nkv_own == nkv) && dk >= 2 && dk % 2 == 0 && dv >= 1,
              "ta_qk_rotate_store: bad sizes nt=%d heads=%d/%d (%d own) widths %d/%d", nt, nh, nkv, nkv_own, dk, dv);
   TA_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dk && (rot == 0 || cs != nullptr) && (style == 0 || style == 1),
@@ -385,11 +391,11 @@ extern "C" int ta_qk_rotate_store(hipStream_t stream, int dtype, void* qkv, int 
   if (dtype == TA_F32)
     qk_rotate_store_kernel<float><<<nt, 256, 0, stream>>>((float*)qkv, stride, bias, rot ? (const float2*)cs : nullptr,
                                                           rot, style, dest, (float*)kcache, (float*)vcache, nh, nkv,
-                                                          nkv_own, dk, dv);
+                                                          nkv_own, dk, dv, dvs);
   else if (dtype == TA_BF16)
     qk_rotate_store_kernel<bf16_t><<<nt, 256, 0, stream>>>((bf16_t*)qkv, stride, bias, rot ? (const float2*)cs : nullptr,
                                                            rot, style, dest, (bf16_t*)kcache, (bf16_t*)vcache, nh, nkv,
-                                                           nkv_own, dk, dv);
+                                                           nkv_own, dk, dv, dvs);
   else return ta_fail("ta_qk_rotate_store: unknown dtype %d", dtype);
   return ta_check_launch("ta_qk_rotate_store");
 }

@@ -1687,7 +1687,9 @@ def qk_rotate_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_di
     """On rows [q | k | v] of ``qkv`` (nh*dk, nkv*dk, nkv*dv columns; q alone without ``own_kv``):
     ``bias`` [columns] float32 is added, the first ``rot`` coordinates of every head of q and k turn by
     ``angles`` [nt, rot/2, 2] ("half": pairs (i, i + rot/2); "interleaved": (2i, 2i + 1)), q goes back
-    in place, k and v are stored at ``dest`` into the cache layer (values of their own width)."""
+    in place, k and v are stored at ``dest`` into the cache layer. The cache's value rows may be wider
+    than the values (vcache [pages, nkv, dvs, PAGE], dvs >= value_dim): the rest of a token's column is
+    zeroed."""
     _dev(qkv, "qkv", contiguous=False)
     nt, stride = _rows2d(qkv, "qkv")
     own = num_kv_heads if own_kv else 0
@@ -1710,14 +1712,17 @@ def qk_rotate_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_di
         if not own_kv:
             raise KernelError("qk_rotate_store: a layer without keys and values of its own stores nothing")
         _dev(dest, "dest", torch.int32); _dev(kcache, "kcache", qkv.dtype); _dev(vcache, "vcache", qkv.dtype)
-        _check_cache_layer("qk_rotate_store", kcache, vcache, num_kv_heads, key_dim, value_dim)
+        store_dim = vcache.shape[2] if vcache.dim() == 4 else -1
+        if store_dim < value_dim:
+            raise KernelError(f"qk_rotate_store: cache value rows of {store_dim} cannot hold values of {value_dim}")
+        _check_cache_layer("qk_rotate_store", kcache, vcache, num_kv_heads, key_dim, store_dim)
         if dest.numel() != nt:
             raise KernelError("qk_rotate_store: dest must hold one entry per token")
     _check(library().ta_qk_rotate_store(
         _stream(), c_int(_code(qkv.dtype)), _ptr(qkv), c_int(stride), _ptr(bias), _ptr(angles), c_int(rot),
         c_int(_ROT_STYLES[style]), _ptr(dest), _ptr(kcache if dest is not None else None),
         _ptr(vcache if dest is not None else None), c_int(nt), c_int(num_heads), c_int(num_kv_heads), c_int(own),
-        c_int(key_dim), c_int(value_dim)))
+        c_int(key_dim), c_int(value_dim), c_int(store_dim if dest is not None else value_dim)))
     return qkv
 
 
@@ -1766,6 +1771,95 @@ def attention_sink(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, nu
         c_int(value_dim), c_float(scale), c_int(window or 0), c_float(softcap or 0.0), c_int(mode),
         _ptr(sink_t), _ptr(gate), c_int(gs)))
     return out
+
+
+def _sink_args(what, q, num_heads, value_dim, softcap, sink, gate):
+    """(softcap, sink mode, sink tensor, gate, gate stride) of the capped softmax's options, checked."""
+    mode, sink_t = 0, None
+    if isinstance(sink, str):
+        if sink != "unit":
+            raise KernelError(f"{what}: unknown sink {sink!r}")
+        mode = 1
+    elif sink is not None:
+        _dev(sink, "sink", torch.float32)
+        if sink.shape != (num_heads,):
+            raise KernelError(f"{what}: sink is {tuple(sink.shape)}, expected {(num_heads,)}")
+        mode, sink_t = 2, sink
+    gs = 0
+    if gate is not None:
+        _dev(gate, "gate", q.dtype, contiguous=False)
+        ng, gs = _rows2d(gate, "gate")
+        if ng != q.shape[0] or gate.shape[1] < num_heads * value_dim:
+            raise KernelError(f"{what}: gate rows are {tuple(gate.shape)}")
+    if softcap is not None and not softcap > 0:
+        raise KernelError(f"{what}: a cap must be positive, got {softcap}")
+    return float(softcap or 0.0), mode, sink_t, gate, gs
+
+
+def attention_rows_sink(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads, num_kv_heads,
+                        head_dim, scale, window=None, softcap=None, sink=None, gate=None, gate_dim=None,
+                        exact=True, through_lds=None):
+    """``attention_rows`` (matrix cores, bfloat16, values as wide as the keys) with the options of
+    ``attention_sink``. gate_dim: columns per head of the gate's rows (the values' own width where the
+    cache pads them to the keys'); out's columns beyond it are not gated. exact: the softmax weights
+    enter the second product as three bfloat16 pieces, so they keep 32 bits. through_lds 0 or 1 (None:
+    1 from 256 rows on)."""
+    if through_lds is None:
+        through_lds = 1 if max_qlen * (num_heads // num_kv_heads) >= 256 and head_dim <= 192 else 0
+    B, qs, os_ = _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads,
+                                 num_kv_heads, head_dim)
+    gd = head_dim if gate_dim is None else int(gate_dim)
+    cap, mode, sink_t, gate, gs = _sink_args("attention_rows_sink", q, num_heads, gd, softcap, sink, gate)
+    _check(library().ta_attention_rows_sink_bf16(
+        _stream(), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache), _ptr(vcache),
+        _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0), c_int(B),
+        c_int(max_qlen), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_float(scale),
+        c_int(window or 0), c_int(int(through_lds)), c_float(cap), c_int(int(exact)), c_int(mode), _ptr(sink_t),
+        _ptr(gate), c_int(gs), c_int(gd)))
+    return out
+
+
+def attention_keys_sink(q, out, kcache, vcache, block_table, cu_q, pos0, max_kv_len, num_heads, num_kv_heads,
+                        head_dim, scale, window=None, softcap=None, sink=None, gate=None, gate_dim=None,
+                        exact=True, units=None, seq_units=None):
+    """``attention_keys`` (single tokens on the matrix cores; q holds rotated heads, the cache the step's
+    keys and values) with the options of ``attention_rows_sink``: the kernel whose four waves take a
+    unit's pages in turn, and the merge, which adds the sink's share and applies the gate."""
+    B, qs, os_ = _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads,
+                                 num_kv_heads, head_dim)
+    if q.shape[0] != B:
+        raise KernelError("attention_keys_sink: every sequence must bring exactly one token")
+    if units is None:
+        lens = [int(p) + 1 for p in pos0.tolist()]
+        if max(lens) > block_table.shape[1] * PAGE:
+            raise KernelError("attention_keys_sink: a sequence is longer than the block table")
+        u, su = plan_key_units(lens, key_unit_count(B, num_kv_heads), tables=block_table.cpu().numpy())
+        units = torch.from_numpy(u).to(q.device)
+        seq_units = torch.from_numpy(su).to(q.device)
+    _dev(units, "units", torch.int32); _dev(seq_units, "seq_units", torch.int32)
+    if units.dim() != 2 or units.shape[1] != UNIT_INTS or tuple(seq_units.shape) != (B, 2) or units.shape[0] < B:
+        raise KernelError(f"attention_keys_sink: units {tuple(units.shape)} / {tuple(seq_units.shape)} for {B} sequences")
+    n_units = units.shape[0]
+    gd = head_dim if gate_dim is None else int(gate_dim)
+    cap, mode, sink_t, gate, gs = _sink_args("attention_keys_sink", q, num_heads, gd, softcap, sink, gate)
+    need = library().ta_attention_keys_scratch
+    need.restype = c_longlong
+    scratch = _scratch_floats(q.device, need(c_int(n_units), c_int(num_heads), c_int(head_dim)))
+    _check(library().ta_attention_keys_sink_bf16(
+        _stream(), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache), _ptr(vcache), _ptr(block_table),
+        c_int(block_table.shape[1]), _ptr(pos0), c_int(B), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim),
+        c_float(scale), c_int(window or 0), _ptr(units), _ptr(seq_units), c_int(n_units), c_int(4), _ptr(scratch),
+        c_float(cap), c_int(int(exact)), c_int(mode), _ptr(sink_t), _ptr(gate), c_int(gs), c_int(gd)))
+    return out
+
+
+def keys_sink_fits(num_heads: int, num_kv_heads: int, head_dim: int) -> bool:
+    """Whether ``attention_keys_sink`` takes this geometry: its four waves merge through 4 * (64 + rows *
+    head size) floats of LDS, which have to fit 64 KB."""
+    if head_dim % 32 or not 32 <= head_dim <= 256:
+        return False
+    group = num_heads // max(num_kv_heads, 1)
+    return (4 * 64 + 4 * min(group, 32) * head_dim) * 4 <= 65536
 
 
 # ------------------------------------------------------------------ short convolution, selective state space
