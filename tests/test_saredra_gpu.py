@@ -120,7 +120,7 @@ def test_routed_gated_experts_part(dtype, geom):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("geom", [(40, 4, True, "silu"), (7, 1, False, None), (300, 2, True, None), (33, 7, False, "silu"),
-                                  (1, 3, True, "silu")])
+                                  (1, 3, True, "silu"), (20, 9, True, None), (70, 8, False, "silu")])
 def test_short_convolution_over_cuts(dtype, geom):
     """Three sequences of unequal lengths in slots that held something else, fed in cuts of many,
     one, two and two tokens: the convolution's memory carries the last inputs (with the
@@ -145,7 +145,7 @@ def test_short_convolution_over_cuts(dtype, geom):
         nt = x.shape[0]
         cu = _t(np.concatenate([[0], np.cumsum([len(r) for r in rows])]), torch.int32)
         out = torch.empty(nt, C, dtype=TD[dtype], device=DEV)
-        K.causal_conv(x, off, C, _t(w), out, state, cu, _t(slots, torch.int32), torch.empty(nt, dtype=torch.int32, device=DEV),
+        K.causal_conv(x, off, C, _t(w), out, state, cu, _t(slots, torch.int32), max(len(r) for r in rows),
                       bias_in=None if bi is None else _t(bi), bias_out=_t(bo), activation=act)
         at = 0
         for i, r in enumerate(rows):

@@ -930,19 +930,81 @@ extern "C" int ta_gla_out(hipStream_t stream, int dtype, const float* o, int par
 }
 
 // ------------------------------------------------------------------ short causal convolution
-// y_t[c] = act(bias_out[c] + sum_j taps[c][j] * u_{t-(K-1-j)}[c]) on a range of columns of the rows
-// of ``in``; u = in + bias_in (a bias that belongs to the projection in front). Inputs before a
+// y_t[c] = act(bias_out[c] + sum_j taps[c][j] * u_{t-(K-1-j)}[c]) on a range of columns of the rows of
+// ``in``; u = in + bias_in (a bias that belongs to the projection in front). Inputs before a
 // sequence's first token of the step come from conv_state [slots, K-1, C] float32 (zero for a new
-// sequence), which `conv_state_update` replaces afterwards by the step's last K-1 inputs.
-// Sums are float32; act 0: none, 1: silu.
+// sequence), which afterwards holds the sequence's last K-1 inputs. Sums are float32; act 0: none,
+// 1: silu.
+#define CONV_MAX_TAPS 8      // taps a thread keeps in registers; more go through the plain kernel
+#define CONV_RUN 16          // tokens a thread of the prompt kernel walks
+
+// the sequence that holds token t: the last b with cu_q[b] <= t
+__device__ __forceinline__ int sequence_of(const int* __restrict__ cu_q, int batch, int t) {
+  int lo = 0, hi = batch - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu_q[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ float conv_act(float v, int act) { return act == 1 ? v / (1.0f + expf(-v)) : v; }
+
+// Prompts: a thread owns one channel and walks CONV_RUN consecutive tokens with the last K - 1 inputs
+// in registers, so every input is read once; where the walk enters another sequence the registers
+// are filled from that sequence's memory. The state is not written here.
+template <typename T, int K>
+__global__ __launch_bounds__(256) void causal_conv_run_kernel(
+    const T* __restrict__ in, int stride, int off, const float* __restrict__ bias_in,
+    const float* __restrict__ taps, const float* __restrict__ bias_out, const float* __restrict__ conv_state,
+    const int* __restrict__ cu_q, const int* __restrict__ slots, int batch, int nt, int C, int act,
+    T* __restrict__ out, int out_stride) {
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int t0 = blockIdx.x * CONV_RUN;
+  if (c >= C || t0 >= nt) return;
+  float w[K], win[K > 1 ? K - 1 : 1];
+#pragma unroll
+  for (int j = 0; j < K; ++j) w[j] = taps[(size_t)c * K + j];
+  const float bi = bias_in ? bias_in[c] : 0.f, bo = bias_out ? bias_out[c] : 0.f;
+  int b = sequence_of(cu_q, batch, t0);
+  int start = cu_q[b], end = cu_q[b + 1];
+  // the K - 1 inputs in front of t0: rows of the step, or the sequence's memory
+#pragma unroll
+  for (int r = 0; r < K - 1; ++r) {
+    const int src = t0 - (K - 1) + r;
+    win[r] = src >= start ? to_f32(in[(size_t)src * stride + off + c]) + bi
+                          : conv_state[((size_t)slots[b] * (K - 1) + (r + (t0 - start))) * C + c];
+  }
+  const int t1 = t0 + CONV_RUN < nt ? t0 + CONV_RUN : nt;
+  for (int t = t0; t < t1; ++t) {
+    if (t >= end) {                      // the next sequence begins: its memory takes the registers
+      ++b;
+      start = end;
+      end = cu_q[b + 1];
+#pragma unroll
+      for (int r = 0; r < K - 1; ++r) win[r] = conv_state[((size_t)slots[b] * (K - 1) + r) * C + c];
+    }
+    const float u = to_f32(in[(size_t)t * stride + off + c]) + bi;
+    float acc = bo;
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) acc = fmaf(w[j], win[j], acc);
+    acc = fmaf(w[K - 1], u, acc);
+#pragma unroll
+    for (int j = 0; j + 1 < K - 1; ++j) win[j] = win[j + 1];
+    if (K > 1) win[K - 2] = u;
+    out[(size_t)t * out_stride + c] = from_f32<T>(conv_act(acc, act));
+  }
+}
+
+// Any number of taps, one thread per (token, channel).
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_kernel(
     const T* __restrict__ in, int stride, int off, const float* __restrict__ bias_in,
     const float* __restrict__ taps, const float* __restrict__ bias_out, const float* __restrict__ conv_state,
-    const int* __restrict__ tok_seq, const int* __restrict__ cu_q, const int* __restrict__ slots, int C, int K,
+    const int* __restrict__ cu_q, const int* __restrict__ slots, int batch, int C, int K,
     int act, T* __restrict__ out, int out_stride) {
   const int t = blockIdx.x;
-  const int b = tok_seq[t];
+  const int b = sequence_of(cu_q, batch, t);
   const int start = cu_q[b];
   const size_t slot = (size_t)slots[b];
   for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
@@ -955,8 +1017,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
       else u = conv_state[(slot * (K - 1) + (K - 1 - (start - src))) * C + c];
       acc = fmaf(taps[(size_t)c * K + j], u, acc);
     }
-    if (act == 1) acc = acc / (1.0f + expf(-acc));
-    out[(size_t)t * out_stride + c] = from_f32<T>(acc);
+    out[(size_t)t * out_stride + c] = from_f32<T>(conv_act(acc, act));
   }
 }
 
@@ -980,39 +1041,93 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(
   }
 }
 
-__global__ void token_sequence_kernel(const int* __restrict__ cu_q, int batch, int* __restrict__ tok_seq) {
+// Steps of single tokens (token b belongs to sequence b): a thread reads its channel's memory, forms
+// the result and writes the memory back moved on by one, all in one kernel.
+template <typename T, int K>
+__global__ __launch_bounds__(256) void causal_conv_step_kernel(
+    const T* __restrict__ in, int stride, int off, const float* __restrict__ bias_in,
+    const float* __restrict__ taps, const float* __restrict__ bias_out, float* __restrict__ conv_state,
+    const int* __restrict__ slots, int C, int act, T* __restrict__ out, int out_stride, int update) {
   const int b = blockIdx.x;
-  for (int t = cu_q[b] + threadIdx.x; t < cu_q[b + 1]; t += blockDim.x) tok_seq[t] = b;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  float* st = conv_state + (size_t)slots[b] * (K - 1) * C + c;
+  float win[K > 1 ? K - 1 : 1];
+#pragma unroll
+  for (int r = 0; r < K - 1; ++r) win[r] = st[(size_t)r * C];
+  const float u = to_f32(in[(size_t)b * stride + off + c]) + (bias_in ? bias_in[c] : 0.f);
+  float acc = bias_out ? bias_out[c] : 0.f;
+#pragma unroll
+  for (int j = 0; j < K - 1; ++j) acc = fmaf(taps[(size_t)c * K + j], win[j], acc);
+  acc = fmaf(taps[(size_t)c * K + K - 1], u, acc);
+  out[(size_t)b * out_stride + c] = from_f32<T>(conv_act(acc, act));
+  if (update) {
+#pragma unroll
+    for (int r = 0; r + 1 < K - 1; ++r) st[(size_t)r * C] = win[r + 1];
+    if (K > 1) st[(size_t)(K - 2) * C] = u;
+  }
 }
 
-// tok_seq [nt] int32 scratch: the sequence of every token of the step (filled here from cu_q).
 // in: [nt, stride] rows, the convolution reads columns off .. off + C; out: [nt, out_stride] rows,
 // columns 0 .. C. taps [C, K] float32; bias_in, bias_out [C] float32 or null; conv_state [slots, K-1, C]
-// float32 (null with K == 1: no memory). update 0: the state is left as it is.
+// float32 (null with K == 1: no memory). update 0: the state is left as it is. max_qlen: the most
+// tokens a sequence brings (1: the single-token kernel).
 extern "C" int ta_causal_conv(hipStream_t stream, int dtype, const void* in, int stride, int off,
                               const float* bias_in, const float* taps, const float* bias_out, float* conv_state,
-                              int* tok_seq, const int* cu_q, const int* slots, int batch, int nt, int C, int K,
+                              const int* cu_q, const int* slots, int batch, int nt, int max_qlen, int C, int K,
                               int act, void* out, int out_stride, int update) {
-  TA_REQUIRE(batch > 0 && batch <= 65535 * 32 && nt >= batch && C >= 1 && K >= 1 && K <= 64,
+  TA_REQUIRE(batch > 0 && batch <= 65535 && nt >= batch && nt <= 65535 * CONV_RUN && C >= 1 && K >= 1 && K <= 64,
              "ta_causal_conv: bad sizes batch=%d nt=%d channels=%d taps=%d", batch, nt, C, K);
   TA_REQUIRE(off >= 0 && stride >= off + C && out_stride >= C && (act == 0 || act == 1),
              "ta_causal_conv: columns %d..%d of rows of %d, out rows of %d, act %d", off, off + C, stride, out_stride, act);
   TA_REQUIRE(K == 1 || conv_state != nullptr, "ta_causal_conv: %d taps need the sequences' memory", K);
-  token_sequence_kernel<<<batch, 256, 0, stream>>>(cu_q, batch, tok_seq);
-  const int cb = (C + 255) / 256 < 64 ? (C + 255) / 256 : 64;
-  dim3 g(nt, cb), gs(batch, cb);
-#define CONV_RUN(T)                                                                                              \
-  do {                                                                                                           \
-    causal_conv_kernel<T><<<g, 256, 0, stream>>>((const T*)in, stride, off, bias_in, taps, bias_out, conv_state, \
-                                                 tok_seq, cu_q, slots, C, K, act, (T*)out, out_stride);         \
-    if (update && K > 1)                                                                                         \
-      conv_state_update_kernel<T><<<gs, 256, 0, stream>>>((const T*)in, stride, off, bias_in, conv_state, cu_q,  \
-                                                          slots, C, K);                                          \
-  } while (0)
-  if (dtype == TA_F32) CONV_RUN(float);
-  else if (dtype == TA_BF16) CONV_RUN(bf16_t);
-  else return ta_fail("ta_causal_conv: unknown dtype %d", dtype);
-#undef CONV_RUN
+  TA_REQUIRE(dtype == TA_F32 || dtype == TA_BF16, "ta_causal_conv: unknown dtype %d", dtype);
+  const int cb = (C + 255) / 256;
+  TA_REQUIRE(cb <= 65535, "ta_causal_conv: too many channels");
+  const bool single = max_qlen == 1 && nt == batch && K <= CONV_MAX_TAPS;
+#define CONV_STEP(T, KK)                                                                                          \
+  causal_conv_step_kernel<T, KK><<<dim3(batch, cb), 256, 0, stream>>>((const T*)in, stride, off, bias_in, taps, \
+                                                                       bias_out, conv_state, slots, C, act, (T*)out, \
+                                                                       out_stride, update)
+#define CONV_RUN_K(T, KK)                                                                                      \
+  causal_conv_run_kernel<T, KK><<<dim3((nt + CONV_RUN - 1) / CONV_RUN, cb), 256, 0, stream>>>(                 \
+      (const T*)in, stride, off, bias_in, taps, bias_out, conv_state, cu_q, slots, batch, nt, C, act, (T*)out, out_stride)
+#define CONV_BY_TAPS(WHAT, T)                \
+  switch (K) {                               \
+    case 1: WHAT(T, 1); break;               \
+    case 2: WHAT(T, 2); break;               \
+    case 3: WHAT(T, 3); break;               \
+    case 4: WHAT(T, 4); break;               \
+    case 5: WHAT(T, 5); break;               \
+    case 6: WHAT(T, 6); break;               \
+    case 7: WHAT(T, 7); break;               \
+    default: WHAT(T, 8); break;              \
+  }
+  if (single) {
+    if (dtype == TA_F32) { CONV_BY_TAPS(CONV_STEP, float) } else { CONV_BY_TAPS(CONV_STEP, bf16_t) }
+    return ta_check_launch("ta_causal_conv");
+  }
+  if (K <= CONV_MAX_TAPS) {
+    if (dtype == TA_F32) { CONV_BY_TAPS(CONV_RUN_K, float) } else { CONV_BY_TAPS(CONV_RUN_K, bf16_t) }
+  } else {
+    const int cbs = cb < 64 ? cb : 64;
+    if (dtype == TA_F32)
+      causal_conv_kernel<float><<<dim3(nt, cbs), 256, 0, stream>>>((const float*)in, stride, off, bias_in, taps, bias_out,
+                                                                   conv_state, cu_q, slots, batch, C, K, act, (float*)out, out_stride);
+    else
+      causal_conv_kernel<bf16_t><<<dim3(nt, cbs), 256, 0, stream>>>((const bf16_t*)in, stride, off, bias_in, taps, bias_out,
+                                                                    conv_state, cu_q, slots, batch, C, K, act, (bf16_t*)out, out_stride);
+  }
+  if (update && K > 1) {
+    const int cbs = cb < 64 ? cb : 64;
+    if (dtype == TA_F32)
+      conv_state_update_kernel<float><<<dim3(batch, cbs), 256, 0, stream>>>((const float*)in, stride, off, bias_in, conv_state, cu_q, slots, C, K);
+    else
+      conv_state_update_kernel<bf16_t><<<dim3(batch, cbs), 256, 0, stream>>>((const bf16_t*)in, stride, off, bias_in, conv_state, cu_q, slots, C, K);
+  }
+#undef CONV_STEP
+#undef CONV_RUN_K
+#undef CONV_BY_TAPS
   return ta_check_launch("ta_causal_conv");
 }
 
@@ -1061,35 +1176,54 @@ extern "C" int ta_ssm_recurrent(hipStream_t stream, int dtype, const void* proj,
 }
 
 // y = (sum of the readout's planes + skip[h] * x) * silu(z), cut into ``groups`` equal parts of the row,
-// each divided by its own root mean square, times w: the gate comes BEFORE the norm. One wave a
-// (token, part); float32 inside. o: [parts, nt, n]; x at column xoff of xs rows, z at zoff of zs rows.
-template <typename T>
-__global__ __launch_bounds__(64) void gated_group_norm_kernel(
+// each divided by its own root mean square, times w: the gate comes BEFORE the norm. A workgroup of
+// THREADS a (token, part); a thread keeps up to GGN_KEEP of the part's columns in registers (all planes
+// asked for at once), so memory is read once; longer parts are formed a second time for the write.
+// float32 inside. o: [parts, nt, n]; x at column xoff of xs rows, z at zoff of zs rows.
+#define GGN_KEEP 8
+template <typename T, int THREADS>
+__global__ __launch_bounds__(THREADS) void gated_group_norm_kernel(
     const float* __restrict__ o, int parts, size_t plane, const T* __restrict__ xs, int x_stride, int xoff,
     const float* __restrict__ skip, int head_dim, const T* __restrict__ zs, int z_stride, int zoff,
     const float* __restrict__ w, float eps, int n, int groups, T* __restrict__ out) {
+  __shared__ float red[THREADS / TA_WAVE];
   const size_t t = blockIdx.x;
   const int g = blockIdx.y, len = n / groups, c0 = g * len;
-  const int lane = threadIdx.x;
-  float ss = 0.f;
-  for (int c = c0 + lane; c < c0 + len; c += 64) {
+  auto value = [&](int c) {
     float y = 0.f;
     for (int p = 0; p < parts; ++p) y += o[p * plane + t * n + c];
     if (skip) y = fmaf(skip[c / head_dim], to_f32(xs[t * x_stride + xoff + c]), y);
     const float z = to_f32(zs[t * z_stride + zoff + c]);
-    y *= z / (1.0f + expf(-z));
+    return y * (z / (1.0f + expf(-z)));
+  };
+  float keep[GGN_KEEP];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < GGN_KEEP; ++i) {
+    const int c = c0 + threadIdx.x + i * THREADS;
+    keep[i] = c < c0 + len ? value(c) : 0.f;
+    ss = fmaf(keep[i], keep[i], ss);
+  }
+  for (int c = c0 + threadIdx.x + GGN_KEEP * THREADS; c < c0 + len; c += THREADS) {
+    const float y = value(c);
     ss = fmaf(y, y, ss);
   }
   ss = wave_sum(ss);
-  const float f = rsqrtf(ss / (float)len + eps);
-  for (int c = c0 + lane; c < c0 + len; c += 64) {
-    float y = 0.f;
-    for (int p = 0; p < parts; ++p) y += o[p * plane + t * n + c];
-    if (skip) y = fmaf(skip[c / head_dim], to_f32(xs[t * x_stride + xoff + c]), y);
-    const float z = to_f32(zs[t * z_stride + zoff + c]);
-    y *= z / (1.0f + expf(-z));
-    out[t * n + c] = from_f32<T>(y * f * (w ? w[c] : 1.f));
+  if (THREADS > TA_WAVE) {
+    if (threadIdx.x % TA_WAVE == 0) red[threadIdx.x / TA_WAVE] = ss;
+    __syncthreads();
+    ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < THREADS / TA_WAVE; ++i) ss += red[i];
   }
+  const float f = rsqrtf(ss / (float)len + eps);
+#pragma unroll
+  for (int i = 0; i < GGN_KEEP; ++i) {
+    const int c = c0 + threadIdx.x + i * THREADS;
+    if (c < c0 + len) out[t * n + c] = from_f32<T>(keep[i] * f * (w ? w[c] : 1.f));
+  }
+  for (int c = c0 + threadIdx.x + GGN_KEEP * THREADS; c < c0 + len; c += THREADS)
+    out[t * n + c] = from_f32<T>(value(c) * f * (w ? w[c] : 1.f));
 }
 
 extern "C" int ta_gated_group_norm(hipStream_t stream, int dtype, const float* o, int parts, const void* xs,
@@ -1101,17 +1235,19 @@ extern "C" int ta_gated_group_norm(hipStream_t stream, int dtype, const float* o
   TA_REQUIRE(skip == nullptr || (head_dim >= 1 && n % head_dim == 0 && x_stride >= xoff + n),
              "ta_gated_group_norm: heads of %d in rows of %d", head_dim, n);
   TA_REQUIRE(z_stride >= zoff + n, "ta_gated_group_norm: gate rows of %d", z_stride);
+  TA_REQUIRE(dtype == TA_F32 || dtype == TA_BF16, "ta_gated_group_norm: unknown dtype %d", dtype);
   if (nt == 0) return 0;
   dim3 g(nt, groups);
   const size_t plane = (size_t)nt * n;
-  if (dtype == TA_F32)
-    gated_group_norm_kernel<float><<<g, 64, 0, stream>>>(o, parts, plane, (const float*)xs, x_stride, xoff, skip,
-                                                         head_dim, (const float*)zs, z_stride, zoff, w, eps, n, groups,
-                                                         (float*)out);
-  else if (dtype == TA_BF16)
-    gated_group_norm_kernel<bf16_t><<<g, 64, 0, stream>>>(o, parts, plane, (const bf16_t*)xs, x_stride, xoff, skip,
-                                                          head_dim, (const bf16_t*)zs, z_stride, zoff, w, eps, n, groups,
-                                                          (bf16_t*)out);
-  else return ta_fail("ta_gated_group_norm: unknown dtype %d", dtype);
+  const int len = n / groups;
+#define GGN(T, TH)                                                                                              \
+  gated_group_norm_kernel<T, TH><<<g, TH, 0, stream>>>(o, parts, plane, (const T*)xs, x_stride, xoff, skip, head_dim, \
+                                                       (const T*)zs, z_stride, zoff, w, eps, n, groups, (T*)out)
+  if (dtype == TA_F32) {
+    if (len <= 256) GGN(float, 64); else GGN(float, 256);
+  } else {
+    if (len <= 256) GGN(bf16_t, 64); else GGN(bf16_t, 256);
+  }
+#undef GGN
   return ta_check_launch("ta_gated_group_norm");
 }

@@ -1867,14 +1867,15 @@ _CONV_ACTS = {None: 0, "silu": 1}
 
 
 def causal_conv(x: torch.Tensor, offset: int, channels: int, taps: torch.Tensor, out: torch.Tensor,
-                conv_state: Optional[torch.Tensor], cu_q: torch.Tensor, slots: torch.Tensor, tok_seq: torch.Tensor,
+                conv_state: Optional[torch.Tensor], cu_q: torch.Tensor, slots: torch.Tensor, max_qlen: int,
                 bias_in: Optional[torch.Tensor] = None, bias_out: Optional[torch.Tensor] = None,
                 activation: Optional[str] = None, update: bool = True) -> torch.Tensor:
     """out[t, c] = act(bias_out[c] + sum_j taps[c, j] * u_(t - K + 1 + j)[c]) per sequence, u = columns
     [offset, offset + channels) of the rows of ``x`` plus ``bias_in``. Inputs before the step's first
     token of a sequence come from conv_state [slots, K - 1, channels] float32 (zero for a new sequence),
     which afterwards holds the sequence's last K - 1 inputs (``update``). taps [channels, K] float32;
-    out [nt, channels] of x's type, not x itself; tok_seq: int32 scratch [nt]."""
+    out [nt, channels] of x's type, not x itself. max_qlen: the most tokens a sequence brings (steps of
+    single tokens take one kernel that also moves the memory on)."""
     _dev(x, "x", contiguous=False); _dev(out, "out", x.dtype, contiguous=False)
     nt, stride = _rows2d(x, "x")
     nto, ostride = _rows2d(out, "out")
@@ -1896,16 +1897,13 @@ def causal_conv(x: torch.Tensor, offset: int, channels: int, taps: torch.Tensor,
         _dev(conv_state, "conv_state", torch.float32)
         if conv_state.dim() != 3 or tuple(conv_state.shape[1:]) != (K - 1, channels):
             raise KernelError(f"causal_conv: state is {tuple(conv_state.shape)}, expected [slots, {K - 1}, {channels}]")
-    _dev(tok_seq, "tok_seq", torch.int32)
-    if tok_seq.numel() < nt:
-        raise KernelError("causal_conv: tok_seq holds one entry per token")
     if out.data_ptr() == x.data_ptr():
         raise KernelError("causal_conv: the result needs rows of its own")
     _check(library().ta_causal_conv(
         _stream(), c_int(_code(x.dtype)), _ptr(x), c_int(stride), c_int(offset), _ptr(bias_in), _ptr(taps),
-        _ptr(bias_out), _ptr(conv_state if K > 1 else None), _ptr(tok_seq), _ptr(cu_q), _ptr(slots), c_int(batch),
-        c_int(nt), c_int(channels), c_int(K), c_int(_CONV_ACTS[activation]), _ptr(out), c_int(ostride),
-        c_int(int(update))))
+        _ptr(bias_out), _ptr(conv_state if K > 1 else None), _ptr(cu_q), _ptr(slots), c_int(batch),
+        c_int(nt), c_int(int(max_qlen)), c_int(channels), c_int(K), c_int(_CONV_ACTS[activation]), _ptr(out),
+        c_int(ostride), c_int(int(update))))
     return out
 
 

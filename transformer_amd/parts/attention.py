@@ -347,7 +347,7 @@ class SinkAttention(Part):
             qkv = ctx.ws.take("attention.conv", (nt, self.qkv_width), self.dtype)
             kernels.causal_conv(proj, 0, self.qkv_width, self.w["conv.weight"], qkv,
                                 cache.layer_state(layer[1]) if s.conv_taps > 1 else None, ctx.cu_q, ctx.slots,
-                                ctx.ws.take("conv.tok_seq", (nt,), torch.int32), bias_in=bias)
+                                ctx.max_qlen, bias_in=bias)
             bias = None
         else:
             qkv = proj[:, :self.qkv_width]

@@ -287,7 +287,7 @@ class StateSpace(Part):
         xbc = ctx.ws.take("state_space.xbc", (nt, self.conv_width), self.dtype)
         kernels.causal_conv(proj, self.inner, self.conv_width, self.w["conv.weight"], xbc,
                             cache.layer_state(layer[1]) if s.taps > 1 else None, ctx.cu_q, ctx.slots,
-                            ctx.ws.take("conv.tok_seq", (nt,), torch.int32), bias_out=self.w["conv.bias"],
+                            ctx.max_qlen, bias_out=self.w["conv.bias"],
                             activation="silu")
         dt = ctx.ws.take("state_space.dt", (nt, H), torch.float32)
         decay = ctx.ws.take("state_space.decay", (nt, H), torch.float32)
