@@ -217,44 +217,63 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
   }
 
   const bool partial = ZERO_TAIL && key0 + TA_PAGE > kv_len;   // unwritten keys hold anything: read them as 0
-  // exact: three passes, each with the bfloat16 rounding of what the passes before left of the weights
-  const int pieces = (XTRA && x.exact) ? 3 : 1;
-#pragma unroll 1
-  for (int piece = 0; piece < pieces; ++piece) {
+  auto values = [&](int mt, int t) {
+    const int kb = 32 * (t / 2) + 16 * (t % 2);
+    Frag a;
+    if (EARLY_V) {
+      a = va[EARLY_V ? mt : 0][t];
+    } else {
+      const bf16_t* vrow = vp + (mt * 32 + j) * VSTR + 4 * h;
+      a.h[0] = *reinterpret_cast<const uint2*>(vrow + kb);
+      a.h[1] = *reinterpret_cast<const uint2*>(vrow + kb + 8);
+    }
+    if (partial) {
+      a.h[0] = zero_from(a.h[0], key0 + kb + 4 * h, kv_len);
+      a.h[1] = zero_from(a.h[1], key0 + kb + 8 + 4 * h, kv_len);
+    }
+    return a;
+  };
+  if (XTRA && x.exact) {
+    // 32-bit weights: three bfloat16 pieces, each the rounding of what the pieces before left; a value
+    // operand is fetched once and multiplied by all three
+    Frag pb3[3][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float a0 = s[t / 2][8 * (t % 2) + 2 * e], a1 = s[t / 2][8 * (t % 2) + 2 * e + 1];
+#pragma unroll
+        for (int piece = 0; piece < 3; ++piece) {
+          const uint32_t two = pack2(a0, a1);
+          pb3[piece][t].w[e] = two;
+          a0 -= __uint_as_float(two << 16);
+          a1 -= __uint_as_float(two & 0xffff0000u);
+        }
+      }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const Frag a = values(mt, t);
+#pragma unroll
+        for (int piece = 0; piece < 3; ++piece)
+          w.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pb3[piece][t].v, w.o[mt], 0, 0, 0);
+      }
+    return;
+  }
   Frag pb[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int i0 = 8 * (t % 2) + 2 * e;
-      const uint32_t two = pack2(s[t / 2][i0], s[t / 2][i0 + 1]);
-      pb[t].w[e] = two;
-      if (XTRA && x.exact) {
-        s[t / 2][i0] -= __uint_as_float(two << 16);
-        s[t / 2][i0 + 1] -= __uint_as_float(two & 0xffff0000u);
-      }
-    }
+    for (int e = 0; e < 4; ++e)
+      pb[t].w[e] = pack2(s[t / 2][8 * (t % 2) + 2 * e], s[t / 2][8 * (t % 2) + 2 * e + 1]);
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const bf16_t* vrow = vp + (mt * 32 + j) * VSTR + 4 * h;
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const int kb = 32 * (t / 2) + 16 * (t % 2);
-      Frag a;
-      if (EARLY_V) {
-        a = va[EARLY_V ? mt : 0][t];
-      } else {
-        a.h[0] = *reinterpret_cast<const uint2*>(vrow + kb);
-        a.h[1] = *reinterpret_cast<const uint2*>(vrow + kb + 8);
-      }
-      if (partial) {
-        a.h[0] = zero_from(a.h[0], key0 + kb + 4 * h, kv_len);
-        a.h[1] = zero_from(a.h[1], key0 + kb + 8 + 4 * h, kv_len);
-      }
+      const Frag a = values(mt, t);
       w.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pb[t].v, w.o[mt], 0, 0, 0);
     }
-  }
-  }
 }
 
 template <int DH>
@@ -1079,7 +1098,9 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
     const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bool all_visible = key0 + TA_PAGE <= kv_len && key0 >= vis_start;   // rows beyond nrows are never written
-    wave_page<DH, DH, TA_PAGE, true, true, XTRA>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h, x);
+    // (with the options the value operands are fetched where they are used: three pieces of weights
+    // and the operands asked for ahead do not fit the registers together)
+    wave_page<DH, DH, TA_PAGE, true, !XTRA, XTRA>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h, x);
   }
 
   // ---- merge the waves: lds = ml[WAVES][32][2] then o[WAVES][nrows][DH]
