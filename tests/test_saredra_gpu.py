@@ -356,7 +356,7 @@ def test_a_sink_takes_its_share(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("geom", [(4, 12, 10, 2, 3), (1, 64, 16, 1, 1), (5, 7, 33, 1, 5), (4, 6, 40, 4, 2), (16, 64, 64, 2, 4),
-                                  (3, 8, 6, 3, 1), (8, 32, 128, 8, 8), (6, 80, 24, 3, 2)])
+                                  (3, 8, 6, 3, 1), (8, 32, 128, 8, 8), (6, 80, 24, 3, 2), (32, 128, 16, 4, 1)])
 def test_state_space_pieces(dtype, geom):
     """Step sizes and decays, the recurrence with the state carried over cuts of many, one and two
     tokens, the skip, the gate before the norm and the norm in parts; three sequences of unequal

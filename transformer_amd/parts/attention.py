@@ -334,7 +334,12 @@ class SinkAttention(Part):
             return [kv, StateNeed((s.conv_taps - 1, self.qkv_width), torch.float32)]
         return kv
 
-    def run(self, h, ctx, cache, layer, writes_cache=True):
+    # with many rows the output projection can add itself to the residual stream (``into``)
+    def can_add(self, nt: int) -> bool:
+        w = self.out_wide if getattr(self, "out_wide", None) is not None else self.w["out.weight"]
+        return adds_in_place(nt, w)
+
+    def run(self, h, ctx, cache, layer, writes_cache=True, into=None):
         s, nt = self.spec, h.shape[0]
         if not s.own_kv and writes_cache:
             raise PartError("a layer without keys and values of its own runs on another layer's cache")
@@ -360,7 +365,7 @@ class SinkAttention(Part):
             o = ctx.ws.take("attention.o", (nt, self.nq * self.dv), self.dtype)
             kernels.attention_sink(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen, self.nq,
                                    self.nkv, self.dk, self.dv, float(s.scale), s.window, s.softcap, sink, gate)
-            return linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta"), None
+            return linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta", into=into), None
         # matrix cores: scores and sums in float32, the softmax weights kept at 32 bits by three pieces
         o = ctx.ws.take("attention.o", (nt, self.nq * self.dk), self.dtype)
         planner = self.step_planner()
@@ -373,7 +378,7 @@ class SinkAttention(Part):
             kernels.attention_rows_sink(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen, self.nq,
                                         self.nkv, self.dk, float(s.scale), s.window, s.softcap, sink, gate, self.dv)
         w = self.out_wide if self.out_wide is not None else self.w["out.weight"]
-        return linear_delta(o, w, ctx.ws, "attention.delta"), None
+        return linear_delta(o, w, ctx.ws, "attention.delta", into=into), None
 
 
 register_part("attention_sink", SinkAttention)
