@@ -271,7 +271,7 @@ def test_capped_sunk_softmax_on_matrix_cores(geom, exact):
     pages = np.array([7, 2, 5, 11, 0, 9, 4, 1, 3, 10, 0, 0])              # ten pages of a table of twelve
     inv = _t(P.rotation_frequencies(rotd)[0]) if rot else None
     got, at = [], 0
-    for n, lds in ((70, 0), (300, 1), (1, None), (1, 0), (28, 0), (1, None), (199, 0)):
+    for n, lds in ((70, 0), (300, 1), (1, None), (1, 0), (28, "vector"), (1, None), (199, 0)):
         p = np.arange(at, at + n)
         qkv = _t(rows[p], TD[dtype])
         angles = K.rope_table(_t(p, torch.int32), inv, torch.empty(n, rot // 2, 2, device=DEV), mag) if rot else None
@@ -282,6 +282,8 @@ def test_capped_sunk_softmax_on_matrix_cores(geom, exact):
         opts = (H, G, dk, scale, window, cap, _t(sinks) if sink == "learned" else sink, _t(gate[p], TD[dtype]) if gated else None, dv)
         if lds is None:
             K.attention_keys_sink(*args, at + 1, *opts, exact=exact)
+        elif lds == "vector":                # the vector kernel over the padded cache: the gate's rows keep their width
+            K.attention_sink(*args, n, H, G, dk, dk, scale, window, cap, opts[6], opts[7], dv)
         else:
             K.attention_rows_sink(*args, n, *opts, exact=exact, through_lds=lds)
         o = _np(o).reshape(n, H, dk)
@@ -723,7 +725,7 @@ def _draw_config(case):
     return cfg, lens, r
 
 
-@pytest.mark.parametrize("first", [5000, 5006, 5012])
+@pytest.mark.parametrize("first", [5000, 5006, 5012, 7020])
 def test_random_configurations_against_the_plain_model(first):
     """float32, the plain model's own routing, every row: a batch of unequal prompts in one step into
     poisoned pages, then eight single tokens each (recorded steps); then the same in bfloat16."""

@@ -30,7 +30,8 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ pos0, int nh, int nkv, int dh, int dv, float scale, int window,
-    float softcap, int sink_mode, const float* __restrict__ sink, const T* __restrict__ gate, int gate_stride) {
+    float softcap, int sink_mode, const float* __restrict__ sink, const T* __restrict__ gate, int gate_stride,
+    int gate_dv) {
   extern __shared__ float smem[];
   const int group = nh / nkv;
   const int b = blockIdx.z, kvh = blockIdx.y;
@@ -158,12 +159,13 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     T* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * dv + lane;
-    const T* gt = gate ? gate + (size_t)(q0 + qi) * gate_stride + (size_t)head * dv + lane : nullptr;
+    // the gate's rows hold gate_dv columns per head (the values' own width where the cache pads them)
+    const T* gt = gate ? gate + (size_t)(q0 + qi) * gate_stride + (size_t)head * gate_dv + lane : nullptr;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
       if (i < nd && 16 * i + lane < dv) {
         float r = acc[i] * inv;
-        if (gt) r *= 1.0f / (1.0f + expf(-to_f32(gt[16 * i])));      // the heads' sigmoid gate
+        if (gt && 16 * i + lane < gate_dv) r *= 1.0f / (1.0f + expf(-to_f32(gt[16 * i])));      // the heads' sigmoid gate
         o[16 * i] = from_f32<T>(r);
       }
   }
@@ -181,11 +183,12 @@ static int attention_generic_launch(hipStream_t stream, int dtype, const void* q
                                     const int* cu_q, const int* pos0, int batch, int max_qlen,
                                     int nh, int nkv, int dh, int dv, float scale, int window,
                                     float softcap = 0.f, int sink_mode = 0, const float* sink = nullptr,
-                                    const void* gate = nullptr, int gate_stride = 0) {
+                                    const void* gate = nullptr, int gate_stride = 0, int gate_dv = 0) {
+  if (gate_dv <= 0) gate_dv = dv;
   TA_REQUIRE(batch >= 0 && max_qlen >= 0, "ta_attention_generic: bad batch=%d max_qlen=%d", batch, max_qlen);
   TA_REQUIRE(sink_mode >= 0 && sink_mode <= 2 && (sink_mode != 2 || sink != nullptr) && softcap >= 0.f,
              "ta_attention_generic: sink mode %d, cap %f", sink_mode, softcap);
-  TA_REQUIRE(gate == nullptr || gate_stride >= nh * dv, "ta_attention_generic: gate rows of %d", gate_stride);
+  TA_REQUIRE(gate == nullptr || (gate_dv <= dv && gate_stride >= nh * gate_dv), "ta_attention_generic: gate rows of %d", gate_stride);
   TA_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "ta_attention_generic: %d heads do not divide into %d kv heads", nh, nkv);
   TA_REQUIRE(dh >= 1 && dh <= 256 && dv >= 1 && dv <= 256,
              "ta_attention_generic: key width %d / value width %d outside [1, 256]", dh, dv);
@@ -200,12 +203,12 @@ static int attention_generic_launch(hipStream_t stream, int dtype, const void* q
     attn_generic_kernel<float><<<g, blk, lds, stream>>>(
         (const float*)q, q_stride, (float*)out, out_stride, (const float*)kcache,
         (const float*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, dv, scale, window,
-        softcap, sink_mode, sink, (const float*)gate, gate_stride);
+        softcap, sink_mode, sink, (const float*)gate, gate_stride, gate_dv);
   else if (dtype == TA_BF16)
     attn_generic_kernel<bf16_t><<<g, blk, lds, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
         (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, dv, scale, window,
-        softcap, sink_mode, sink, (const bf16_t*)gate, gate_stride);
+        softcap, sink_mode, sink, (const bf16_t*)gate, gate_stride, gate_dv);
   else
     return ta_fail("ta_attention_generic: unknown dtype %d", dtype);
   return ta_check_launch("ta_attention_generic");
@@ -232,15 +235,16 @@ extern "C" int ta_attention_generic_dv(hipStream_t stream, int dtype, const void
 
 // The same with the options of a capped, sunk and gated softmax: softcap > 0: score <- softcap *
 // tanh(score / softcap) after the scale; sink_mode 1: the denominator holds one more term exp(0);
-// 2: exp(sink[head]) (float32 [nh]); gate: rows [nt, >= nh*dv] whose sigmoid multiplies the result.
+// 2: exp(sink[head]) (float32 [nh]); gate: rows [nt, >= nh*gate_dv] whose sigmoid multiplies the first gate_dv
+// columns of every head of the result (gate_dv <= dv; 0: dv).
 extern "C" int ta_attention_generic_sink(hipStream_t stream, int dtype, const void* q, int q_stride,
                                          void* out, int out_stride, const void* kcache,
                                          const void* vcache, const int* block_table, int max_blocks,
                                          const int* cu_q, const int* pos0, int batch, int max_qlen,
                                          int nh, int nkv, int dh, int dv, float scale, int window,
                                          float softcap, int sink_mode, const float* sink, const void* gate,
-                                         int gate_stride) {
+                                         int gate_stride, int gate_dv) {
   return attention_generic_launch(stream, dtype, q, q_stride, out, out_stride, kcache, vcache, block_table,
                                   max_blocks, cu_q, pos0, batch, max_qlen, nh, nkv, dh, dv, scale, window,
-                                  softcap, sink_mode, sink, gate, gate_stride);
+                                  softcap, sink_mode, sink, gate, gate_stride, gate_dv);
 }

@@ -1728,11 +1728,13 @@ def qk_rotate_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_di
 
 def attention_sink(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads, num_kv_heads, key_dim,
                    value_dim, scale, window=None, softcap: Optional[float] = None, sink=None,
-                   gate: Optional[torch.Tensor] = None):
+                   gate: Optional[torch.Tensor] = None, gate_dim: Optional[int] = None):
     """``attention_generic_dv`` with the options of a capped, sunk and gated softmax. softcap: score <-
     softcap * tanh(score / softcap) after the scale. sink: None; "unit": the denominator holds one more
     term exp(0) = 1; a float32 tensor [heads]: one more term exp(sink[head]). gate: rows [nt, >= heads *
-    value_dim] of q's type whose sigmoid multiplies the result element by element."""
+    value_dim] of q's type whose sigmoid multiplies the result element by element. gate_dim: columns per
+    head of the gate's rows where that is less than value_dim (a cache whose value rows are padded): the
+    result's columns beyond it are not gated."""
     _dev(q, "q", contiguous=False); _dev(out, "out", q.dtype, contiguous=False)
     nt, qs = _rows2d(q, "q")
     nto, os_ = _rows2d(out, "out")
@@ -1746,30 +1748,16 @@ def attention_sink(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, nu
     B = pos0.numel()
     if cu_q.numel() != B + 1 or block_table.dim() != 2 or block_table.shape[0] != B:
         raise KernelError("attention: cu_q / pos0 / block_table disagree about the batch size")
-    mode, sink_t = 0, None
-    if isinstance(sink, str):
-        if sink != "unit":
-            raise KernelError(f"attention: unknown sink {sink!r}")
-        mode = 1
-    elif sink is not None:
-        _dev(sink, "sink", torch.float32)
-        if sink.shape != (num_heads,):
-            raise KernelError(f"attention: sink is {tuple(sink.shape)}, expected {(num_heads,)}")
-        mode, sink_t = 2, sink
-    gs = 0
-    if gate is not None:
-        _dev(gate, "gate", q.dtype, contiguous=False)
-        ng, gs = _rows2d(gate, "gate")
-        if ng != nt or gate.shape[1] < num_heads * value_dim:
-            raise KernelError(f"attention: gate rows are {tuple(gate.shape)}")
-    if softcap is not None and not softcap > 0:
-        raise KernelError(f"attention: a cap must be positive, got {softcap}")
+    gd = value_dim if gate_dim is None else int(gate_dim)
+    if not 1 <= gd <= value_dim:
+        raise KernelError(f"attention: gate columns per head {gd} outside [1, {value_dim}]")
+    cap, mode, sink_t, gate, gs = _sink_args("attention", q, num_heads, gd, softcap, sink, gate)
     _check(library().ta_attention_generic_sink(
         _stream(), c_int(_code(q.dtype)), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache),
         _ptr(vcache), _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0),
         c_int(B), c_int(max_qlen), c_int(num_heads), c_int(num_kv_heads), c_int(key_dim),
-        c_int(value_dim), c_float(scale), c_int(window or 0), c_float(softcap or 0.0), c_int(mode),
-        _ptr(sink_t), _ptr(gate), c_int(gs)))
+        c_int(value_dim), c_float(scale), c_int(window or 0), c_float(cap), c_int(mode),
+        _ptr(sink_t), _ptr(gate), c_int(gs), c_int(gd)))
     return out
 
 

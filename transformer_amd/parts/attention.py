@@ -304,11 +304,16 @@ class SinkAttention(Part):
     # bfloat16 with a key width the matrix-core kernels take and values no wider than the keys: the
     # cache keeps value rows of the keys' width (the rest zero), so that the kernels for equal widths
     # serve prompts and single tokens, and the output projection reads the heads' rows through a copy
-    # of its matrix with zero columns in the same places (as ``NormedAttention`` does). Everything else
-    # (float32, other widths) runs the vector-ALU kernel on values of their own width.
+    # of its matrix with zero columns in the same places (as ``NormedAttention`` does). This depends on
+    # the type and the two widths alone, which a layer shares with the readers of its cache. Everything
+    # else (float32, other widths) runs the vector-ALU kernel on values of their own width.
+    def _pads_values(self) -> bool:
+        return self.dtype == torch.bfloat16 and self.dk % 32 == 0 and 32 <= self.dk <= 256 and self.dv <= self.dk
+
     def _on_matrix_cores(self) -> bool:
-        return (self.dtype == torch.bfloat16 and self.dk % 32 == 0 and 32 <= self.dk <= 256 and self.dv <= self.dk
-                and self.width % 8 == 0 and self.qkv_width % 8 == 0)      # rows of q start on 16 bytes
+        # ... and rows of q that start on 16 bytes; a layer whose rows do not reads the padded cache
+        # through the vector-ALU kernel
+        return self._pads_values() and self.width % 8 == 0 and self.qkv_width % 8 == 0
 
     def step_planner(self):
         if self._on_matrix_cores() and kernels.keys_sink_fits(self.nq, self.nkv, self.dk):
@@ -318,7 +323,7 @@ class SinkAttention(Part):
     def bind(self, tensors):
         super().bind(tensors)
         self.out_wide = None
-        if self._on_matrix_cores() and self.dv < self.dk and tensors["out.weight"].is_cuda:
+        if self._pads_values() and self.dv < self.dk and tensors["out.weight"].is_cuda:
             w = tensors["out.weight"]
             wide = torch.zeros(w.shape[0], self.nq, self.dk, dtype=w.dtype, device=w.device)
             wide[:, :, :self.dv] = w.view(w.shape[0], self.nq, self.dv)
@@ -328,7 +333,7 @@ class SinkAttention(Part):
         s = self.spec
         # cache_window None: the layer's own window; 0: every token is kept; else that many
         window = s.window if s.cache_window is None else (s.cache_window or None)
-        kv = KVNeed(self.nkv, self.dk, window, self.dk if self._on_matrix_cores() else self.dv)
+        kv = KVNeed(self.nkv, self.dk, window, self.dk if self._pads_values() else self.dv)
         if s.conv_taps > 1:
             from ..cache.storage import StateNeed
             return [kv, StateNeed((s.conv_taps - 1, self.qkv_width), torch.float32)]
@@ -361,23 +366,26 @@ class SinkAttention(Part):
                                 s.rot_style, meta.dest if (writes_cache and s.own_kv) else None, kc, vc)
         sink = self.w["sink"] if s.sink == "learned" else s.sink
         gate = proj[:, self.qkv_width:] if s.out_gate else None
+        w = self.out_wide if self.out_wide is not None else self.w["out.weight"]
         if not self._on_matrix_cores():
-            o = ctx.ws.take("attention.o", (nt, self.nq * self.dv), self.dtype)
+            vd = self.dk if self._pads_values() else self.dv          # the width of the cache's value rows
+            o = ctx.ws.take("attention.o", (nt, self.nq * vd), self.dtype)
             kernels.attention_sink(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen, self.nq,
-                                   self.nkv, self.dk, self.dv, float(s.scale), s.window, s.softcap, sink, gate)
-            return linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta", into=into), None
+                                   self.nkv, self.dk, vd, float(s.scale), s.window, s.softcap, sink, gate, self.dv)
+            return linear_delta(o, w, ctx.ws, "attention.delta", into=into), None
         # matrix cores: scores and sums in float32, the softmax weights kept at 32 bits by three pieces
         o = ctx.ws.take("attention.o", (nt, self.nq * self.dk), self.dtype)
         planner = self.step_planner()
-        if ctx.all_single and planner is not None:
-            plan = meta.plans.get(planner, {})
+        # (the units of work are planned with the step's tables for the layer that owns the cache; a
+        # reader whose lender has none takes the prompt kernel, which serves single tokens too)
+        plan = meta.plans.get(planner) if planner is not None else None
+        if ctx.all_single and plan:
             kernels.attention_keys_sink(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_kv_len, self.nq,
                                         self.nkv, self.dk, float(s.scale), s.window, s.softcap, sink, gate, self.dv,
                                         units=plan.get("units"), seq_units=plan.get("seq_units"))
         else:
             kernels.attention_rows_sink(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen, self.nq,
                                         self.nkv, self.dk, float(s.scale), s.window, s.softcap, sink, gate, self.dv)
-        w = self.out_wide if self.out_wide is not None else self.w["out.weight"]
         return linear_delta(o, w, ctx.ws, "attention.delta", into=into), None
 
 
