@@ -8,6 +8,10 @@
 // and every row's running maximum, sum and output are updated in that order, so
 // a row's result depends only on its own query and keys: not on the batch, not
 // on how the tokens were cut into steps, not on which pages hold the keys.
+//
+// Options (all off in the plain entry points): scores capped by cap * tanh(score / cap); one more
+// term in the softmax denominator that has no value (a "sink": exp(0), or exp of a learned number
+// per head); the result multiplied by the sigmoid of a gate row.
 #include "common.h"
 
 #define ROWS 16

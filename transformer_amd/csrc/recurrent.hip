@@ -14,6 +14,15 @@
 //   `gla_decay` forms alpha for all tokens at once, `gla_recurrent` walks a sequence's tokens in
 //   order with S in registers; `gla_out` applies the per-head RMS norm and the output gate.
 //
+// Selective state space ("ssm"): per head a matrix state S [N][P] with one decay per (token, head),
+//     dt_t = softplus(raw_t + bias), S_t = exp(-exp(A) dt_t) S_{t-1} + dt_t B_t x_t^T, o_t = S_t^T C_t
+//   `ssm_steps` forms step sizes and decays, the recurrence is `gla_recurrent` with q = C, k = B, v = x
+//   (the heads of a group read the same B and C), `gated_group_norm` adds D x, gates and norms.
+//
+// Short causal convolution (`causal_conv`): per channel over a sequence's tokens, with the last
+//   inputs of every sequence kept between steps; used in front of the state space and by the
+//   attention variant that convolves its q, k and v.
+//
 // All state, decays, gates and sums are float32; tokens are walked in the same order however a
 // sequence was cut into steps, so the cut does not change a bit of the result.
 #include "common.h"
